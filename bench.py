@@ -1,0 +1,170 @@
+"""Benchmark of the block-local grid update on one MI355X.
+
+One "step" = one pass of the network body over one synthetic batch: ``outer`` x (stencil step,
+LayerNorm) forward and, for training workloads, the same chain backward, called through the C
+ABI on preallocated device buffers (inputs resident in HBM before the clock starts).
+Prints ONE JSON line with the headline metric, the roofline of the dominant kernel and the
+CPU baseline (the reference-style torch path, timed on this machine's host cores).
+"""
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor peak
+
+
+def gpu_run(wl, steps, warmup):
+    import torch
+
+    from gridnet_amd.configs import make_inputs
+    from gridnet_amd.runner import BodyRunner
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    t = {k: v.to(dev) for k, v in make_inputs(wl, seed=0).items()}
+    run = BodyRunner(t["weight"], t["bias"], t["scale"], t["gamma"], t["beta"], wl.batch, wl.inner,
+                     wl.outer, wl.block_size, wl.activation, wl.normalize, backward=wl.backward)
+
+    def one_step():
+        run.forward(t["x0"])
+        if wl.backward:
+            run.backward(t["grad_out"])
+
+    for _ in range(warmup):
+        one_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        one_step()
+    torch.cuda.synchronize()
+    wall = (time.perf_counter() - t0) / steps
+
+    # per-entry-point device time: events recorded on the stream the kernels are launched on
+    # (torch's current stream is the one handed to the C ABI), in a separate instrumented pass
+    spans = {}
+    pending = []
+
+    def hook(name, phase):
+        ev = torch.cuda.Event(enable_timing=True)
+        ev.record(torch.cuda.current_stream(dev))
+        pending.append((name, phase, ev))
+
+    run.on_launch = hook
+    reps = max(2, min(steps, 5))
+    for _ in range(reps):
+        one_step()
+    torch.cuda.synchronize()
+    run.on_launch = None
+    for (name, p0, e0), (_, p1, e1) in zip(pending[0::2], pending[1::2]):
+        assert p0 == 0 and p1 == 1
+        spans.setdefault(name, []).append(e0.elapsed_time(e1) * 1e-3)
+    kernel_s = {k: sum(v) / len(v) for k, v in spans.items()}
+    return wall, kernel_s
+
+
+def cpu_baseline(wl, budget_s=25.0):
+    """The reference-style pure-torch path (block loop + gather; oracle.ref_style) composed with
+    F.layer_norm, forward + autograd backward, on a bounded sample of the workload."""
+    import torch
+
+    from gridnet_amd.configs import make_inputs
+    from oracle.network import network_forward
+    from oracle.ref_style import gridnet_step_ref
+
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    grid, batch = min(wl.grid, 64), min(wl.batch, 32)
+    t = make_inputs(wl, seed=0, batch=batch, grid=grid)
+    params = [t[k].requires_grad_(wl.backward) for k in ("weight", "bias", "scale", "gamma", "beta")]
+    x0 = t["x0"].requires_grad_(wl.backward)
+
+    def once():
+        y = network_forward(*params, x0, wl.inner, 1, wl.block_size, wl.activation, wl.normalize,
+                            step_fn=gridnet_step_ref)
+        if wl.backward:
+            torch.autograd.grad(y, params + [x0], t["grad_out"])
+
+    tiny = make_inputs(wl, seed=0, batch=2, grid=16)  # warm-up: thread pool, allocator
+    network_forward(*[tiny[k] for k in ("weight", "bias", "scale", "gamma", "beta")], tiny["x0"],
+                    wl.inner, 1, wl.block_size, wl.activation, wl.normalize, step_fn=gridnet_step_ref)
+    times = []
+    start = time.perf_counter()
+    while len(times) < 3 and (time.perf_counter() - start < budget_s or not times):
+        t0 = time.perf_counter()
+        once()
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    cu = batch * grid ** 3 * wl.inner
+    return {
+        "value": cu / med,
+        "unit": "cell-updates/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"one outer step {'fwd+bwd' if wl.backward else 'fwd'} of a {grid}^3 grid, "
+                  f"batch {batch}, bs {wl.block_size}, inner {wl.inner} "
+                  f"(median of {len(times)}, {med:.2f} s each)",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="C3")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (no collectives, no sharding); "
+                 "use --gpus 1")
+    from gridnet_amd.configs import WORKLOADS
+
+    wl = WORKLOADS[args.workload]
+    wall, kernel_s = gpu_run(wl, args.steps, args.warmup)
+    bytes_ = wl.algorithmic_bytes()
+    dominant = max(kernel_s, key=lambda k: kernel_s[k])
+    dom_s = kernel_s[dominant]
+    achieved = bytes_[dominant] / dom_s / 1e9
+    out = {
+        "metric": "cell-updates/s fwd+bwd, 64^3 grid 8^3 blocks batch 32; % of HBM roofline",
+        "value": wl.cell_updates / wall,
+        "unit": "cell-updates/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": wall * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": wl.name, "activation": wl.activation, "normalize": wl.normalize,
+                   "pass": "fwd+bwd" if wl.backward else "fwd"},
+        "hbm_roofline_frac_whole_step": bytes_["total"] / wall / (HBM_PEAK_GBS * 1e9),
+        "entry_point_ms": {k: v * 1e3 for k, v in kernel_s.items()},
+        "roofline": {
+            "bound": "hbm",
+            "kernel": dominant,
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": None,
+        },
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(wl)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,316 @@
+// Per-sample LayerNorm over all grid cells with elementwise affine, forward and backward.
+//
+// The callers of the grid update run torch.nn.LayerNorm((M,N,K)) after every outer step
+// (gridnet/scripts/train_mnist.py:54,64; gridnet/scripts/train_imagenet.py:67,86), so one
+// "sample" is a whole grid: n = M*N*K cells (262 144 at 64^3), far more than a workgroup
+// holds.  Each sample is therefore cut into chunks of 4096 cells, one workgroup per chunk:
+//
+//   forward   ln_partial_stats : per chunk (mean, M2) with M2 centred on the chunk's own mean
+//             ln_apply         : every workgroup merges its sample's chunk statistics in a
+//                                fixed order (exact pairwise-combination formula, no
+//                                E[x^2]-mean^2 cancellation) and normalises its chunk
+//   backward  ln_bwd_partial   : per chunk sum(g) and sum(g*xhat), g = dy*gamma
+//             ln_bwd_finalize  : per sample means of the two
+//             ln_bwd_apply     : one thread owns 4 adjacent cells for ALL samples, so dgamma
+//                                and dbeta are reduced over the batch in registers, without
+//                                atomics and in a fixed order
+//
+// Every reduction has a fixed order, so results are bitwise reproducible.
+
+#include "common.h"
+#include "launch.h"
+
+namespace gridnet {
+
+namespace {
+
+constexpr int kLnThreads = 256;
+constexpr int kLnPerThread = 16;
+constexpr int kLnChunk = kLnThreads * kLnPerThread;  // cells per workgroup
+
+template <typename T> struct alignas(4 * sizeof(T)) Vec4 { T v[4]; };
+
+// Load this thread's 16 cells of a chunk; cells past `n` read as `fill` and are not counted.
+// Layout: 4 rounds; in a round the 256 threads read 256 consecutive groups of 4 cells.
+template <typename T, bool VEC>
+__device__ __forceinline__ void load_chunk(const T *p, long start, long n, int tid, T (&r)[kLnPerThread]) {
+#pragma unroll
+    for (int round = 0; round < 4; ++round) {
+        const long at = start + ((long)round * kLnThreads + tid) * 4;
+        if (VEC) {
+            if (at < n) {  // n % 4 == 0: the whole group is in range
+                const Vec4<T> q = *reinterpret_cast<const Vec4<T> *>(p + at);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) r[round * 4 + e] = q.v[e];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) r[round * 4 + e] = T(0);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) r[round * 4 + e] = (at + e < n) ? p[at + e] : T(0);
+        }
+    }
+}
+
+template <typename T, bool VEC>
+__device__ __forceinline__ void store_chunk(T *p, long start, long n, int tid, const T (&r)[kLnPerThread]) {
+#pragma unroll
+    for (int round = 0; round < 4; ++round) {
+        const long at = start + ((long)round * kLnThreads + tid) * 4;
+        if (VEC) {
+            if (at < n) {
+                Vec4<T> q;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) q.v[e] = r[round * 4 + e];
+                *reinterpret_cast<Vec4<T> *>(p + at) = q;
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (at + e < n) p[at + e] = r[round * 4 + e];
+        }
+    }
+}
+
+__device__ __forceinline__ bool cell_valid(long start, long n, int tid, int i) {
+    return start + ((long)(i / 4) * kLnThreads + tid) * 4 + (i % 4) < n;
+}
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kLnThreads) void ln_partial_stats(const T *__restrict__ x,
+                                                               T *__restrict__ partial, long n,
+                                                               int nchunk) {
+    __shared__ T red[kLnThreads / kWave];
+    const int tid = threadIdx.x, chunk = blockIdx.x, b = blockIdx.y;
+    const long start = (long)chunk * kLnChunk;
+    const long count = min((long)kLnChunk, n - start);
+    T r[kLnPerThread];
+    load_chunk<T, VEC>(x + (long)b * n, start, n, tid, r);
+    T s = T(0);
+#pragma unroll
+    for (int i = 0; i < kLnPerThread; ++i) s += r[i];  // out-of-range cells hold 0
+    const T mean = block_sum(s, red, tid, kLnThreads) / T(count);
+    T q = T(0);
+#pragma unroll
+    for (int i = 0; i < kLnPerThread; ++i) {
+        const T d = r[i] - mean;
+        q += cell_valid(start, n, tid, i) ? d * d : T(0);
+    }
+    const T m2 = block_sum(q, red, tid, kLnThreads);
+    if (tid == 0) {
+        partial[((long)b * nchunk + chunk) * 2 + 0] = mean;
+        partial[((long)b * nchunk + chunk) * 2 + 1] = m2;
+    }
+}
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kLnThreads) void ln_apply(const T *__restrict__ x,
+                                                       const T *__restrict__ gamma,
+                                                       const T *__restrict__ beta,
+                                                       const T *__restrict__ partial,
+                                                       T *__restrict__ y, T *__restrict__ mean_out,
+                                                       T *__restrict__ rstd_out, long n, int nchunk,
+                                                       T eps) {
+    __shared__ T red[kLnThreads / kWave];
+    const int tid = threadIdx.x, chunk = blockIdx.x, b = blockIdx.y;
+    const T *ps = partial + (long)b * nchunk * 2;
+    // merge the chunk statistics of this sample: mean = sum(c_i m_i)/n,
+    // M2 = sum(M2_i + c_i (m_i - mean)^2)
+    T s = T(0);
+    for (int c = tid; c < nchunk; c += kLnThreads) {
+        const long cnt = min((long)kLnChunk, n - (long)c * kLnChunk);
+        s += T(cnt) * ps[c * 2];
+    }
+    const T mean = block_sum(s, red, tid, kLnThreads) / T(n);
+    T q = T(0);
+    for (int c = tid; c < nchunk; c += kLnThreads) {
+        const long cnt = min((long)kLnChunk, n - (long)c * kLnChunk);
+        const T d = ps[c * 2] - mean;
+        q += ps[c * 2 + 1] + T(cnt) * d * d;
+    }
+    const T var = block_sum(q, red, tid, kLnThreads) / T(n);
+    const T rstd = T(1) / sqrt(var + eps);
+    if (chunk == 0 && tid == 0) {
+        mean_out[b] = mean;
+        rstd_out[b] = rstd;
+    }
+    const long start = (long)chunk * kLnChunk;
+    T r[kLnPerThread], gm[kLnPerThread], bt[kLnPerThread];
+    load_chunk<T, VEC>(x + (long)b * n, start, n, tid, r);
+    load_chunk<T, VEC>(gamma, start, n, tid, gm);
+    load_chunk<T, VEC>(beta, start, n, tid, bt);
+#pragma unroll
+    for (int i = 0; i < kLnPerThread; ++i) r[i] = (r[i] - mean) * rstd * gm[i] + bt[i];
+    store_chunk<T, VEC>(y + (long)b * n, start, n, tid, r);
+}
+
+template <typename T, bool VEC>
+__global__ __launch_bounds__(kLnThreads) void ln_bwd_partial(const T *__restrict__ dy,
+                                                             const T *__restrict__ x,
+                                                             const T *__restrict__ gamma,
+                                                             const T *__restrict__ mean,
+                                                             const T *__restrict__ rstd,
+                                                             T *__restrict__ partial, long n,
+                                                             int nchunk) {
+    __shared__ T red[kLnThreads / kWave];
+    const int tid = threadIdx.x, chunk = blockIdx.x, b = blockIdx.y;
+    const long start = (long)chunk * kLnChunk;
+    const T mu = mean[b], rs = rstd[b];
+    T g[kLnPerThread], xv[kLnPerThread], gm[kLnPerThread];
+    load_chunk<T, VEC>(dy + (long)b * n, start, n, tid, g);
+    load_chunk<T, VEC>(x + (long)b * n, start, n, tid, xv);
+    load_chunk<T, VEC>(gamma, start, n, tid, gm);
+    T s1 = T(0), s2 = T(0);
+#pragma unroll
+    for (int i = 0; i < kLnPerThread; ++i) {
+        const T gi = g[i] * gm[i];  // out-of-range cells: dy = 0 -> no contribution
+        s1 += gi;
+        s2 += gi * ((xv[i] - mu) * rs);
+    }
+    s1 = block_sum(s1, red, tid, kLnThreads);
+    s2 = block_sum(s2, red, tid, kLnThreads);
+    if (tid == 0) {
+        partial[((long)b * nchunk + chunk) * 2 + 0] = s1;
+        partial[((long)b * nchunk + chunk) * 2 + 1] = s2;
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kLnThreads) void ln_bwd_finalize(const T *__restrict__ partial,
+                                                              T *__restrict__ sample_means, long n,
+                                                              int nchunk) {
+    __shared__ T red[kLnThreads / kWave];
+    const int tid = threadIdx.x, b = blockIdx.x;
+    const T *ps = partial + (long)b * nchunk * 2;
+    T s1 = T(0), s2 = T(0);
+    for (int c = tid; c < nchunk; c += kLnThreads) {
+        s1 += ps[c * 2];
+        s2 += ps[c * 2 + 1];
+    }
+    s1 = block_sum(s1, red, tid, kLnThreads);
+    s2 = block_sum(s2, red, tid, kLnThreads);
+    if (tid == 0) {
+        sample_means[b * 2 + 0] = s1 / T(n);
+        sample_means[b * 2 + 1] = s2 / T(n);
+    }
+}
+
+template <typename T, int VEC, bool ACCUM>
+__global__ __launch_bounds__(kLnThreads) void ln_bwd_apply(
+    const T *__restrict__ dy, const T *__restrict__ x, const T *__restrict__ gamma,
+    const T *__restrict__ mean, const T *__restrict__ rstd, const T *__restrict__ sample_means,
+    T *__restrict__ dx, T *__restrict__ dgamma, T *__restrict__ dbeta, int B, long n) {
+    const long at = ((long)blockIdx.x * kLnThreads + threadIdx.x) * VEC;
+    if (at >= n) return;
+    T gm[VEC], dg[VEC], dbt[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+        gm[e] = gamma[at + e];
+        dg[e] = T(0);
+        dbt[e] = T(0);
+    }
+    struct alignas(sizeof(T) * VEC) Pack { T v[VEC]; };
+#pragma unroll 4
+    for (int b = 0; b < B; ++b) {
+        const T mu = mean[b], rs = rstd[b];
+        const T c1 = sample_means[b * 2], c2 = sample_means[b * 2 + 1];
+        const Pack d = *reinterpret_cast<const Pack *>(dy + (long)b * n + at);
+        const Pack xv = *reinterpret_cast<const Pack *>(x + (long)b * n + at);
+        Pack o;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            const T xh = (xv.v[e] - mu) * rs;
+            dg[e] += d.v[e] * xh;
+            dbt[e] += d.v[e];
+            o.v[e] = rs * (d.v[e] * gm[e] - c1 - xh * c2);
+        }
+        *reinterpret_cast<Pack *>(dx + (long)b * n + at) = o;
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+        if (ACCUM) {
+            dgamma[at + e] += dg[e];
+            dbeta[at + e] += dbt[e];
+        } else {
+            dgamma[at + e] = dg[e];
+            dbeta[at + e] = dbt[e];
+        }
+    }
+}
+
+inline int chunks_of(long n) { return (int)((n + kLnChunk - 1) / kLnChunk); }
+
+template <typename T> bool aligned4(const void *p) { return ((uintptr_t)p % (4 * sizeof(T))) == 0; }
+
+template <typename T> int forward_t(const LayerNormArgs &a, hipStream_t st) {
+    const int nchunk = chunks_of(a.n);
+    T *partial = (T *)a.workspace;
+    const bool vec = a.n % 4 == 0 && aligned4<T>(a.x) && aligned4<T>(a.y) && aligned4<T>(a.gamma) &&
+                     aligned4<T>(a.beta);
+    dim3 grid(nchunk, a.B), block(kLnThreads);
+    if (vec) {
+        hipLaunchKernelGGL((ln_partial_stats<T, true>), grid, block, 0, st, (const T *)a.x, partial,
+                           a.n, nchunk);
+        hipLaunchKernelGGL((ln_apply<T, true>), grid, block, 0, st, (const T *)a.x,
+                           (const T *)a.gamma, (const T *)a.beta, partial, (T *)a.y, (T *)a.mean,
+                           (T *)a.rstd, a.n, nchunk, (T)a.eps);
+    } else {
+        hipLaunchKernelGGL((ln_partial_stats<T, false>), grid, block, 0, st, (const T *)a.x, partial,
+                           a.n, nchunk);
+        hipLaunchKernelGGL((ln_apply<T, false>), grid, block, 0, st, (const T *)a.x,
+                           (const T *)a.gamma, (const T *)a.beta, partial, (T *)a.y, (T *)a.mean,
+                           (T *)a.rstd, a.n, nchunk, (T)a.eps);
+    }
+    return check_launch("layernorm_forward");
+}
+
+template <typename T> int backward_t(const LayerNormArgs &a, hipStream_t st) {
+    const int nchunk = chunks_of(a.n);
+    T *partial = (T *)a.workspace;
+    T *sample_means = partial + (long)a.B * nchunk * 2;
+    const bool vec = a.n % 4 == 0 && aligned4<T>(a.x) && aligned4<T>(a.dy) && aligned4<T>(a.gamma) &&
+                     aligned4<T>(a.dx);
+    const bool accum = (a.flags & GRIDNET_OVERWRITE_PARAMS) == 0;
+    dim3 grid(nchunk, a.B), block(kLnThreads);
+    if (vec)
+        hipLaunchKernelGGL((ln_bwd_partial<T, true>), grid, block, 0, st, (const T *)a.dy,
+                           (const T *)a.x, (const T *)a.gamma, (const T *)a.mean_in,
+                           (const T *)a.rstd_in, partial, a.n, nchunk);
+    else
+        hipLaunchKernelGGL((ln_bwd_partial<T, false>), grid, block, 0, st, (const T *)a.dy,
+                           (const T *)a.x, (const T *)a.gamma, (const T *)a.mean_in,
+                           (const T *)a.rstd_in, partial, a.n, nchunk);
+    hipLaunchKernelGGL((ln_bwd_finalize<T>), dim3(a.B), block, 0, st, partial, sample_means, a.n,
+                       nchunk);
+#define GRIDNET_LN_APPLY(V, ACC)                                                                   \
+    hipLaunchKernelGGL((ln_bwd_apply<T, V, ACC>),                                                  \
+                       dim3((unsigned)((a.n + (long)kLnThreads * V - 1) / ((long)kLnThreads * V))), \
+                       block, 0, st, (const T *)a.dy, (const T *)a.x, (const T *)a.gamma,          \
+                       (const T *)a.mean_in, (const T *)a.rstd_in, sample_means, (T *)a.dx,        \
+                       (T *)a.dgamma, (T *)a.dbeta, a.B, a.n)
+    if (vec) {
+        if (accum) GRIDNET_LN_APPLY(4, true); else GRIDNET_LN_APPLY(4, false);
+    } else {
+        if (accum) GRIDNET_LN_APPLY(1, true); else GRIDNET_LN_APPLY(1, false);
+    }
+#undef GRIDNET_LN_APPLY
+    return check_launch("layernorm_backward");
+}
+
+}  // namespace
+
+size_t layernorm_workspace(int dtype, int B, long n) {
+    const size_t elt = dtype == GRIDNET_F64 ? 8 : 4;
+    return ((size_t)B * chunks_of(n) * 2 + (size_t)B * 2) * elt;
+}
+
+int layernorm_forward(const LayerNormArgs &a, hipStream_t st) {
+    return a.dtype == GRIDNET_F64 ? forward_t<double>(a, st) : forward_t<float>(a, st);
+}
+
+int layernorm_backward(const LayerNormArgs &a, hipStream_t st) {
+    return a.dtype == GRIDNET_F64 ? backward_t<double>(a, st) : backward_t<float>(a, st);
+}
+
+}  // namespace gridnet

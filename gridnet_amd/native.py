@@ -1,0 +1,109 @@
+"""ctypes binding of libgridnet_hip.so (the C ABI declared in include/gridnet_hip.h).
+
+The library is the product; there is no fallback.  If it has not been built this module
+raises ImportError on import, which the dispatcher in ``gridnet_amd/__init__.py`` treats the
+way the reference treats a missing extension (gridnet/__init__.py:14-18) -- and calling an op
+on a HIP tensor without it raises instead of silently running something else.
+"""
+
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libgridnet_hip.so")
+
+F32, F64 = 0, 1
+OVERWRITE_PARAMS = 1
+OVERWRITE_DX = 2
+OVERWRITE = 3
+
+EXPORTS = (
+    "gridnet_hip_version",
+    "gridnet_hip_last_error",
+    "gridnet_hip_activation_id",
+    "gridnet_hip_forward",
+    "gridnet_hip_backward_workspace_bytes",
+    "gridnet_hip_backward",
+    "gridnet_hip_layernorm_workspace_bytes",
+    "gridnet_hip_layernorm_forward",
+    "gridnet_hip_layernorm_backward",
+)
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m gridnet_amd.build` "
+            "(hipcc --offload-arch=gfx950)"
+        )
+    try:
+        lib = ctypes.CDLL(LIB_PATH)
+    except OSError as exc:  # unresolved HIP runtime, wrong arch, ...
+        raise ImportError(f"cannot load {LIB_PATH}: {exc}") from exc
+    p, i, d, l, z = ctypes.c_void_p, ctypes.c_int, ctypes.c_double, ctypes.c_long, ctypes.c_size_t
+    lib.gridnet_hip_version.restype = i
+    lib.gridnet_hip_version.argtypes = []
+    lib.gridnet_hip_last_error.restype = ctypes.c_char_p
+    lib.gridnet_hip_last_error.argtypes = []
+    lib.gridnet_hip_activation_id.restype = i
+    lib.gridnet_hip_activation_id.argtypes = [ctypes.c_char_p]
+    lib.gridnet_hip_forward.restype = i
+    lib.gridnet_hip_forward.argtypes = [i, p, p, p, p, p, i, i, i, i, i, i, d, i, i, p]
+    lib.gridnet_hip_backward_workspace_bytes.restype = z
+    lib.gridnet_hip_backward_workspace_bytes.argtypes = [i, i, i, i, i, i, i, i]
+    lib.gridnet_hip_backward.restype = i
+    lib.gridnet_hip_backward.argtypes = [i, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, d, i, i, i,
+                                         p, z, p]
+    lib.gridnet_hip_layernorm_workspace_bytes.restype = z
+    lib.gridnet_hip_layernorm_workspace_bytes.argtypes = [i, i, l]
+    lib.gridnet_hip_layernorm_forward.restype = i
+    lib.gridnet_hip_layernorm_forward.argtypes = [i, p, p, p, p, p, p, i, l, d, p, z, p]
+    lib.gridnet_hip_layernorm_backward.restype = i
+    lib.gridnet_hip_layernorm_backward.argtypes = [i, p, p, p, p, p, p, p, p, i, l, i, p, z, p]
+    return lib
+
+
+lib = _load()
+
+
+def last_error() -> str:
+    return lib.gridnet_hip_last_error().decode()
+
+
+def check(status: int) -> None:
+    if status != 0:
+        raise RuntimeError(last_error())
+
+
+def activation_id(name: str) -> int:
+    act = lib.gridnet_hip_activation_id(str(name).encode())
+    if act < 0:
+        raise RuntimeError(last_error())  # "unknown activation function: X"
+    return act
+
+
+def dtype_id(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return F32
+    if t.dtype == torch.float64:
+        return F64
+    raise RuntimeError(f"gridnet_hip supports float32 and float64 tensors, got {t.dtype}")
+
+
+def check_input(t: torch.Tensor, name: str) -> None:
+    """The reference binding's CHECK_INPUT (src/gridnet_cuda.cpp:6-10), same messages."""
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+
+
+def current_stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def workspace(nbytes: int, device) -> torch.Tensor:
+    """Scratch from torch's caching allocator (stream-ordered reuse, no hipMalloc per call)."""
+    return torch.empty(max(int(nbytes), 1), dtype=torch.uint8, device=device)

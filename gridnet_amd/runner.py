@@ -1,0 +1,110 @@
+"""Allocation-free driver of the network body on the C ABI: ``outer`` x (step, LayerNorm)
+forward, then the same chain backward, on preallocated buffers.
+
+This is what a training loop that owns its buffers (or a captured HIP graph) calls; the
+autograd ops in ``backend_cuda``/``layernorm`` do the same launches with torch-managed
+memory.  Order of operations: gridnet/scripts/train_mnist.py:62-64.
+"""
+
+import torch
+
+from . import native as _n
+
+
+class BodyRunner:
+    def __init__(self, weight, bias, scale, gamma, beta, batch: int, inner: int, outer: int,
+                 block_size: int, activation: str = "leaky_relu", normalize: bool = False,
+                 eps: float = 1e-5, ln_eps: float = 1e-5, backward: bool = True):
+        self.w, self.b, self.r, self.gamma, self.beta = weight, bias, scale, gamma, beta
+        self.B, (self.M, self.N, self.K) = batch, bias.shape
+        self.inner, self.outer, self.bs = inner, outer, block_size
+        self.act = _n.activation_id(activation)
+        self.normalize, self.eps, self.ln_eps = int(normalize), eps, ln_eps
+        self.dt = _n.dtype_id(weight)
+        dev, dtype = weight.device, weight.dtype
+        n = bias.numel()
+        self.n = n
+        shape = (batch, self.M, self.N, self.K)
+        keep = outer if backward else 1
+        # h[j]: input of outer step j (h[outer] = result); s[j]: its output before the norm
+        self.h = [torch.empty(shape, device=dev, dtype=dtype) for _ in range(keep + 1)]
+        self.s = [torch.empty(shape, device=dev, dtype=dtype) for _ in range(keep)]
+        self.mean = torch.empty(keep, batch, device=dev, dtype=dtype)
+        self.rstd = torch.empty(keep, batch, device=dev, dtype=dtype)
+        self.ln_ws_bytes = _n.lib.gridnet_hip_layernorm_workspace_bytes(self.dt, batch, n)
+        self.ln_ws = _n.workspace(self.ln_ws_bytes, dev)
+        self.has_backward = backward
+        if backward:
+            self.ga = torch.empty(shape, device=dev, dtype=dtype)
+            self.gb = torch.empty(shape, device=dev, dtype=dtype)
+            self.dw = torch.empty_like(weight)
+            self.db = torch.empty_like(bias)
+            self.dr = torch.empty_like(bias)
+            self.dgamma = torch.empty_like(bias)
+            self.dbeta = torch.empty_like(bias)
+            self.bw_ws_bytes = _n.lib.gridnet_hip_backward_workspace_bytes(
+                self.dt, batch, self.M, self.N, self.K, inner, block_size, self.normalize)
+            self.bw_ws = _n.workspace(self.bw_ws_bytes, dev)
+        self.on_launch = None  # optional hook(name, phase) for per-kernel timing
+
+    def _mark(self, name, phase):
+        if self.on_launch is not None:
+            self.on_launch(name, phase)
+
+    def step_forward(self, x, y, stream):
+        self._mark("step_fwd", 0)
+        _n.check(_n.lib.gridnet_hip_forward(
+            self.dt, self.w.data_ptr(), self.b.data_ptr(), self.r.data_ptr(), x.data_ptr(),
+            y.data_ptr(), self.B, self.M, self.N, self.K, self.inner, self.bs, self.eps,
+            self.normalize, self.act, stream))
+        self._mark("step_fwd", 1)
+
+    def norm_forward(self, x, y, j, stream):
+        self._mark("ln_fwd", 0)
+        _n.check(_n.lib.gridnet_hip_layernorm_forward(
+            self.dt, x.data_ptr(), self.gamma.data_ptr(), self.beta.data_ptr(), y.data_ptr(),
+            self.mean[j].data_ptr(), self.rstd[j].data_ptr(), self.B, self.n, self.ln_eps,
+            self.ln_ws.data_ptr(), self.ln_ws_bytes, stream))
+        self._mark("ln_fwd", 1)
+
+    def forward(self, x0):
+        """Returns the buffer holding the result (valid until the next call)."""
+        stream = _n.current_stream(self.w)
+        self.h[0].copy_(x0)
+        if self.has_backward:
+            for j in range(self.outer):
+                self.step_forward(self.h[j], self.s[j], stream)
+                self.norm_forward(self.s[j], self.h[j + 1], j, stream)
+            return self.h[self.outer]
+        for j in range(self.outer):  # forward only: ping-pong, nothing is kept
+            self.step_forward(self.h[j % 2], self.s[0], stream)
+            self.norm_forward(self.s[0], self.h[(j + 1) % 2], 0, stream)
+        return self.h[self.outer % 2]
+
+    def backward(self, grad_out):
+        """Backward of the last ``forward``.  Returns (dweight, dbias, dscale, dgamma, dbeta, dx0);
+        parameter gradients are summed over the outer steps (shared parameters)."""
+        assert self.has_backward
+        stream = _n.current_stream(self.w)
+        g = grad_out
+        for j in reversed(range(self.outer)):
+            flags = _n.OVERWRITE_PARAMS if j == self.outer - 1 else 0
+            self._mark("ln_bwd", 0)
+            _n.check(_n.lib.gridnet_hip_layernorm_backward(
+                self.dt, g.data_ptr(), self.s[j].data_ptr(), self.gamma.data_ptr(),
+                self.mean[j].data_ptr(), self.rstd[j].data_ptr(), self.ga.data_ptr(),
+                self.dgamma.data_ptr(), self.dbeta.data_ptr(), self.B, self.n, flags,
+                self.ln_ws.data_ptr(), self.ln_ws_bytes, stream))
+            self._mark("ln_bwd", 1)
+            self._mark("step_bwd", 0)
+            # dx is fully written every time; parameter gradients are written by the first
+            # call and accumulated into by the later ones (parameters are shared)
+            _n.check(_n.lib.gridnet_hip_backward(
+                self.dt, self.w.data_ptr(), self.b.data_ptr(), self.r.data_ptr(),
+                self.h[j].data_ptr(), self.ga.data_ptr(), self.dw.data_ptr(), self.db.data_ptr(),
+                self.dr.data_ptr(), self.gb.data_ptr(), self.B, self.M, self.N, self.K, self.inner,
+                self.bs, self.eps, self.normalize, self.act, flags | _n.OVERWRITE_DX,
+                self.bw_ws.data_ptr(), self.bw_ws_bytes, stream))
+            self._mark("step_bwd", 1)
+            g = self.gb
+        return self.dw, self.db, self.dr, self.dgamma, self.dbeta, self.gb

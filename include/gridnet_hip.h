@@ -1,0 +1,121 @@
+/*
+ * gridnet_hip.h -- C ABI of libgridnet_hip.so: the block-local grid update of gridnet
+ * (3x3x3 per-cell-weight stencil with stale halos, its backward, and the per-sample
+ * LayerNorm the callers interleave with it) as hand-written HIP kernels for gfx950.
+ *
+ * Conventions shared by every entry point
+ *   - All pointers are DEVICE pointers into memory the caller owns.  The library never
+ *     allocates, frees, retains or synchronises; every call only enqueues kernels on
+ *     `stream` (a hipStream_t passed as void*, NULL = the default stream).
+ *   - Tensors are dense, row-major, K fastest: weight [27, M, N, K] with tap index
+ *     t = 9a + 3b + c addressing neighbour (i+a-1, j+b-1, k+c-1); bias, scale [M, N, K];
+ *     activations [B, M, N, K].  (gridnet/__init__.py:42-49, gridnet/backend_torch.py:283-298)
+ *   - `dtype` is GRIDNET_F32 or GRIDNET_F64 and applies to every tensor of the call.
+ *   - Return value 0 = enqueued.  Non-zero = nothing was enqueued; the message is
+ *     available from gridnet_hip_last_error() on the calling thread.
+ */
+#ifndef GRIDNET_HIP_H
+#define GRIDNET_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum gridnet_dtype { GRIDNET_F32 = 0, GRIDNET_F64 = 1 };
+
+/* Activation ids; the names are the strings the reference dispatches on
+ * (src/activations.h:6-17, gridnet/backend_torch.py:270-280). */
+enum gridnet_activation {
+    GRIDNET_ACT_RELU = 0,
+    GRIDNET_ACT_LEAKY_RELU = 1, /* slope 0.01 */
+    GRIDNET_ACT_SILU = 2,
+    GRIDNET_ACT_TANH = 3
+};
+
+/* Status codes. */
+enum gridnet_status {
+    GRIDNET_OK = 0,
+    GRIDNET_ERR_ARGUMENT = 1,   /* bad shape / block size / pointer / dtype */
+    GRIDNET_ERR_ACTIVATION = 2, /* "unknown activation function: X" (src/activations.h:16) */
+    GRIDNET_ERR_ITERATIONS = 3, /* "cannot backprop through more than 32 inner iterations"
+                                   (src/gridnet_cuda_kernels.cu:836) */
+    GRIDNET_ERR_WORKSPACE = 4,  /* workspace missing or too small */
+    GRIDNET_ERR_LAUNCH = 5      /* hipGetLastError() after the launch */
+};
+
+/* Flags for the backward entry points. */
+enum gridnet_flags {
+    /* Default (0): every gradient output is ACCUMULATED into, as the reference's kernels do
+     * with atomicAdd into buffers its wrapper zero-filled (gridnet/backend_cuda.py:78-81,
+     * src/gridnet_cuda_kernels.cu:424-449).  With a flag set, that output need not be
+     * initialised: it is fully written. */
+    GRIDNET_OVERWRITE_PARAMS = 1, /* dweight, dbias, dscale (LayerNorm: dgamma, dbeta) */
+    GRIDNET_OVERWRITE_DX = 2,     /* dx (LayerNorm: dx is always fully written) */
+    GRIDNET_OVERWRITE = 3
+};
+
+/* Library build id (monotonic integer) -- lets a binding check it loaded what it expects. */
+int gridnet_hip_version(void);
+
+/* Thread-local message of the last non-zero status returned on this thread ("" if none). */
+const char *gridnet_hip_last_error(void);
+
+/* Map an activation name to its id, or -1 (and set the reference's message
+ * "unknown activation function: <name>").  Replaces APPLY_ACTIVATION, src/activations.h:6-17. */
+int gridnet_hip_activation_id(const char *name);
+
+/*
+ * One outer step, forward.  Replaces gridnet_cuda_forward, src/gridnet_cuda_kernels.cu:736-784
+ * (bound as `forward`, src/gridnet_cuda.cpp:61-89,190).
+ *   y is fully overwritten.  inner >= 0.  block_size in {4, 8} and must divide M, N and K.
+ *   eps/normalize: per-window normalisation (x-mean)/(std+eps) over the (bs+2)^3 window.
+ */
+int gridnet_hip_forward(int dtype, const void *weight, const void *bias, const void *scale,
+                        const void *x, void *y, int B, int M, int N, int K, int inner,
+                        int block_size, double eps, int normalize, int activation,
+                        void *stream);
+
+/*
+ * Scratch needed by gridnet_hip_backward for this problem (bytes, may be 0).
+ */
+size_t gridnet_hip_backward_workspace_bytes(int dtype, int B, int M, int N, int K, int inner,
+                                            int block_size, int normalize);
+
+/*
+ * One outer step, backward.  Replaces gridnet_cuda_backward, src/gridnet_cuda_kernels.cu:786-851
+ * (bound as `backward`, src/gridnet_cuda.cpp:91-131,191).  Recomputes the inner forward
+ * from x; inner <= 32.  dweight [27,M,N,K], dbias, dscale [M,N,K] are summed over the batch;
+ * dx [B,M,N,K].  `workspace` must hold gridnet_hip_backward_workspace_bytes() bytes (contents
+ * need no initialisation; 256-byte aligned).
+ */
+int gridnet_hip_backward(int dtype, const void *weight, const void *bias, const void *scale,
+                         const void *x, const void *dy, void *dweight, void *dbias,
+                         void *dscale, void *dx, int B, int M, int N, int K, int inner,
+                         int block_size, double eps, int normalize, int activation, int flags,
+                         void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Per-sample LayerNorm over all n = M*N*K cells with elementwise affine, the op the callers
+ * place after every outer step (torch.nn.LayerNorm((M,N,K)): gridnet/scripts/train_mnist.py:54,64,
+ * gridnet/scripts/train_imagenet.py:67,86).  y = (x-mean)*rstd*gamma + beta, biased variance,
+ * rstd = 1/sqrt(var+eps).  mean, rstd: [B] outputs kept for the backward.
+ */
+size_t gridnet_hip_layernorm_workspace_bytes(int dtype, int B, long n);
+
+int gridnet_hip_layernorm_forward(int dtype, const void *x, const void *gamma, const void *beta,
+                                  void *y, void *mean, void *rstd, int B, long n, double eps,
+                                  void *workspace, size_t workspace_bytes, void *stream);
+
+/* dx [B,n] (always fully written); dgamma, dbeta [n] summed over the batch (accumulated
+ * unless GRIDNET_OVERWRITE_PARAMS). */
+int gridnet_hip_layernorm_backward(int dtype, const void *dy, const void *x, const void *gamma,
+                                   const void *mean, const void *rstd, void *dx, void *dgamma,
+                                   void *dbeta, int B, long n, int flags, void *workspace,
+                                   size_t workspace_bytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GRIDNET_HIP_H */

@@ -1,0 +1,115 @@
+"""CPU checks of the drop-in boundary: the library loads, exports what the header declares,
+answers its host-only entry points, and the Python shim has the reference's call surface."""
+
+import ctypes
+import inspect
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "gridnet_hip.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(gridnet_hip_\w+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    names = declared_symbols()
+    for want in ("gridnet_hip_forward", "gridnet_hip_backward", "gridnet_hip_layernorm_forward",
+                 "gridnet_hip_layernorm_backward", "gridnet_hip_last_error"):
+        assert want in names
+
+
+def test_library_exports_every_declared_symbol():
+    from gridnet_amd import native
+
+    lib = ctypes.CDLL(native.LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(lib, name), f"{name} declared in include/gridnet_hip.h but not exported"
+    assert set(native.EXPORTS) == set(declared_symbols())
+
+
+def test_host_only_entry_points():
+    from gridnet_amd import native
+
+    assert native.lib.gridnet_hip_version() >= 1
+    assert [native.activation_id(n) for n in ("relu", "leaky_relu", "silu", "tanh")] == [0, 1, 2, 3]
+    with pytest.raises(RuntimeError, match="unknown activation function: gelu"):
+        native.activation_id("gelu")
+    # argument validation happens before anything touches a device
+    rc = native.lib.gridnet_hip_forward(0, 8, 8, 8, 8, 8, 2, 12, 8, 8, 1, 8, 1e-5, 0, 0, None)
+    assert rc == 1 and "incompatible" in native.last_error()
+    rc = native.lib.gridnet_hip_forward(0, 8, 8, 8, 8, 8, 2, 8, 8, 8, 1, 2, 1e-5, 0, 0, None)
+    assert rc == 1 and "block_size" in native.last_error()
+    rc = native.lib.gridnet_hip_backward(0, 8, 8, 8, 8, 8, 8, 8, 8, 8, 2, 8, 8, 8, 33, 8, 1e-5, 0,
+                                         0, 0, None, 0, None)
+    assert rc == 3
+    assert native.last_error() == "cannot backprop through more than 32 inner iterations"
+    rc = native.lib.gridnet_hip_forward(0, 8, 8, 8, 8, 8, 2, 8, 8, 8, 1, 8, 1e-5, 0, 7, None)
+    assert rc == 2 and "unknown activation function" in native.last_error()
+    assert native.lib.gridnet_hip_layernorm_workspace_bytes(0, 32, 64 ** 3) == (32 * 64 * 2 + 64) * 4
+    rc = native.lib.gridnet_hip_layernorm_forward(0, 8, 8, 8, 8, 8, 8, 4, 4096, 1e-5, None, 0, None)
+    assert rc == 4 and "workspace" in native.last_error()
+
+
+def test_shim_has_the_reference_call_surface():
+    """Positional signatures of src/gridnet_cuda.cpp:61-72, 91-106, 133-141, 160-171."""
+    import gridnet_cuda
+
+    assert list(inspect.signature(gridnet_cuda.forward).parameters) == [
+        "weight", "bias", "scale", "initActivations", "outActivations", "innerIterations",
+        "blockSize", "eps", "normalize", "activation"]
+    assert list(inspect.signature(gridnet_cuda.backward).parameters) == [
+        "weight", "bias", "scale", "initActivations", "outGrads", "weightGradOut", "biasGradOut",
+        "scaleGradOut", "activationsGradOut", "innerIterations", "blockSize", "eps", "normalize",
+        "activation"]
+    assert len(inspect.signature(gridnet_cuda.forward_gated).parameters) == 7
+    assert len(inspect.signature(gridnet_cuda.backward_gated).parameters) == 10
+
+
+def test_shim_rejects_host_tensors_like_the_reference_binding():
+    import torch
+
+    import gridnet_cuda
+
+    t = torch.zeros(1, 8, 8, 8)
+    w = torch.zeros(27, 8, 8, 8)
+    p = torch.zeros(8, 8, 8)
+    with pytest.raises(RuntimeError, match="weight must be a CUDA tensor"):
+        gridnet_cuda.forward(w, p, p, t, t.clone(), 1, 8, 1e-5, False, "silu")
+
+
+def test_dispatcher_never_falls_back():
+    import torch
+
+    import gridnet_amd
+
+    w, p, t = torch.zeros(27, 8, 8, 8), torch.zeros(8, 8, 8), torch.zeros(1, 8, 8, 8)
+    with pytest.raises(NotImplementedError, match="HIP devices only"):
+        gridnet_amd.gridnet_step(w, p, p, t, 1, 8)
+
+
+def test_autograd_op_keeps_the_reference_contract():
+    import torch
+
+    from gridnet_amd.backend_cuda import GridnetCudaOp
+
+    params = list(inspect.signature(GridnetCudaOp.forward).parameters)
+    assert params == ["ctx", "weight", "bias", "residual_scale", "init_activations", "inner_iters",
+                      "block_size", "eps", "normalize", "activation"]
+    w, p = torch.zeros(27, 8, 8, 8), torch.zeros(8, 8, 8)
+    # gridnet/backend_cuda.py:20-22 and :51-52
+    with pytest.raises(AssertionError, match="incompatible"):
+        GridnetCudaOp.apply(w, p, p, torch.zeros(1, 8, 8, 8), 1, 3, 1e-5, False, "silu")
+    with pytest.raises(AssertionError, match="invalid"):
+        GridnetCudaOp.apply(w[:26], p, p, torch.zeros(1, 8, 8, 8), 1, 8, 1e-5, False, "silu")
+    with pytest.raises(AssertionError, match="mismatching dtypes"):
+        GridnetCudaOp.apply(w, p.double(), p, torch.zeros(1, 8, 8, 8), 1, 8, 1e-5, False, "silu")
+    empty = torch.zeros(0, 8, 8, 8)
+    out = GridnetCudaOp.apply(w, p, p, empty, 1, 8, 1e-5, False, "silu")
+    assert out.shape == empty.shape and out.data_ptr() != empty.data_ptr() or out.numel() == 0

@@ -1,0 +1,177 @@
+"""GPU parity of one outer step (forward and all four gradients) against the CPU oracle,
+called through the reference's own op interface (GridnetCudaOp.apply -> gridnet_cuda ->
+C ABI).  Bar: rtol 1e-4 / atol 1e-5 in fp32 against the oracle evaluated in fp64 on the same
+fp32 inputs; fp64 runs are held to 1e-9."""
+
+import pytest
+import torch
+
+from oracle.fast import gridnet_step_fast
+from oracle.manual import gridnet_step_backward_manual
+
+from helpers import ATOL, RTOL, assert_close, make_acts, make_params
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def run_op(w, b, r, x, gy, inner, bs, eps, normalize, activation):
+    from gridnet_amd.backend_cuda import GridnetCudaOp
+
+    leaves = [t.to(DEV).requires_grad_(True) for t in (w, b, r, x)]
+    y = GridnetCudaOp.apply(*leaves, inner, bs, eps, normalize, activation)
+    if gy is None:
+        return y.detach().cpu(), None
+    grads = torch.autograd.grad(y, leaves, gy.to(DEV))
+    return y.detach().cpu(), [g.cpu() for g in grads]
+
+
+def oracle(w, b, r, x, gy, inner, bs, eps, normalize, activation):
+    w, b, r, x = (t.double() for t in (w, b, r, x))
+    y = gridnet_step_fast(w, b, r, x, inner, bs, eps, normalize, activation)
+    if gy is None:
+        return y, None
+    grads = gridnet_step_backward_manual(w, b, r, x, gy.double(), inner, bs, eps, normalize,
+                                         activation)
+    return y, list(grads)
+
+
+def compare(case, dtype=torch.float32, all_randn=False, rtol=RTOL, atol=ATOL, batch=2):
+    shape, bs, inner, normalize, activation = case
+    print(f"case shape={shape} bs={bs} inner={inner} normalize={normalize} act={activation} "
+          f"dtype={dtype} B={batch}", flush=True)
+    w, b, r = make_params(shape, seed=11, dtype=dtype, all_randn=all_randn)
+    x = make_acts(batch, shape, seed=12, dtype=dtype)
+    gy = make_acts(batch, shape, seed=13, dtype=dtype)
+    y, grads = run_op(w, b, r, x, gy, inner, bs, 1e-5, normalize, activation)
+    ey, egrads = oracle(w, b, r, x, gy, inner, bs, 1e-5, normalize, activation)
+    assert_close(y, ey, rtol, atol, "y")
+    for name, g, e in zip(("dweight", "dbias", "dscale", "dx"), grads, egrads):
+        assert_close(g, e, rtol, atol, name)
+
+
+# the reference's own matrix (gridnet/backend_cuda_test.py:11-17, 64-71), plus more depths
+MATRIX = [
+    ((16, 16, 16), 8, 2, True, "silu"),
+    ((16, 16, 16), 8, 1, True, "silu"),
+    ((32, 64, 128), 8, 2, True, "silu"),
+    ((32, 64, 128), 4, 2, True, "silu"),
+    ((32, 16, 8), 4, 2, False, "silu"),
+    ((32, 16, 8), 8, 2, False, "silu"),
+    ((16, 16, 16), 8, 2, False, "leaky_relu"),
+    ((32, 64, 128), 8, 2, False, "leaky_relu"),
+    ((32, 64, 128), 4, 2, False, "leaky_relu"),
+    ((16, 8, 24), 8, 4, False, "leaky_relu"),
+    ((16, 8, 24), 4, 8, False, "tanh"),
+    ((8, 8, 8), 8, 0, False, "relu"),
+    ((8, 16, 8), 4, 3, False, "relu"),
+    ((8, 16, 8), 8, 5, True, "tanh"),
+    ((8, 16, 8), 4, 3, True, "relu"),
+]
+
+
+@pytest.mark.parametrize("case", MATRIX, ids=lambda c: "-".join(map(str, c)).replace(" ", ""))
+def test_step_parity_fp32(case):
+    compare(case)
+
+
+@pytest.mark.parametrize("case", MATRIX[:6] + MATRIX[9:11],
+                         ids=lambda c: "-".join(map(str, c)).replace(" ", ""))
+def test_step_parity_fp64(case):
+    compare(case, dtype=torch.float64, rtol=1e-9, atol=1e-9)
+
+
+@pytest.mark.parametrize("case", MATRIX[:6], ids=lambda c: "-".join(map(str, c)).replace(" ", ""))
+def test_reference_matrix_at_reference_bounds(case):
+    """All-N(0,1) parameters as in gridnet/backend_cuda_test.py:25-36: values reach the
+    hundreds, so the reference's own absolute bound (2e-4) is applied relative to scale."""
+    shape, bs, inner, normalize, activation = case
+    w, b, r = make_params(shape, seed=21, all_randn=True)
+    x = make_acts(2, shape, seed=22)
+    y, _ = run_op(w, b, r, x, None, inner, bs, 1e-5, normalize, activation)
+    ey, _ = oracle(w, b, r, x, None, inner, bs, 1e-5, normalize, activation)
+    scale = max(1.0, ey.abs().max().item())
+    assert (y.double() - ey).abs().max().item() < 2e-4 * scale
+
+
+@pytest.mark.parametrize("batch", [1, 3, 33])
+@pytest.mark.parametrize("bs", [4, 8])
+def test_batch_sizes(batch, bs):
+    compare(((16, 8, 8), bs, 2, False, "leaky_relu"), batch=batch)
+
+
+@pytest.mark.parametrize("inner", [16, 32])
+def test_deep_inner_iterations(inner):
+    # small weights keep 32 residual updates tame
+    shape, bs = (8, 8, 16), 8
+    w, b, r = make_params(shape, seed=3)
+    w, r = w * 0.3, r * 0.2
+    x, gy = make_acts(2, shape, seed=4), make_acts(2, shape, seed=5)
+    y, grads = run_op(w, b, r, x, gy, inner, bs, 1e-5, False, "tanh")
+    ey, eg = oracle(w, b, r, x, gy, inner, bs, 1e-5, False, "tanh")
+    assert_close(y, ey, what="y")
+    for name, g, e in zip(("dweight", "dbias", "dscale", "dx"), grads, eg):
+        assert_close(g, e, what=name)
+
+
+def test_empty_batch_returns_a_clone():
+    from gridnet_amd.backend_cuda import GridnetCudaOp
+
+    shape = (8, 8, 8)
+    w, b, r = (t.to(DEV) for t in make_params(shape))
+    x = torch.zeros(0, *shape, device=DEV)
+    y = GridnetCudaOp.apply(w, b, r, x, 2, 8, 1e-5, False, "silu")
+    assert y.shape == x.shape
+
+
+def test_error_paths_raise_like_the_reference():
+    import gridnet_cuda
+    from gridnet_amd.backend_cuda import GridnetCudaOp
+
+    shape = (8, 8, 8)
+    w, b, r = (t.to(DEV) for t in make_params(shape))
+    x = make_acts(2, shape).to(DEV)
+    with pytest.raises(RuntimeError, match="unknown activation function: gelu"):
+        GridnetCudaOp.apply(w, b, r, x, 1, 8, 1e-5, False, "gelu")
+    with pytest.raises(RuntimeError, match="initActivations must be contiguous"):
+        gridnet_cuda.forward(w, b, r, x.transpose(1, 2), torch.empty_like(x), 1, 8, 1e-5, False,
+                             "silu")
+    with pytest.raises(RuntimeError, match="bias must be a CUDA tensor"):
+        gridnet_cuda.forward(w, b.cpu(), r, x, torch.empty_like(x), 1, 8, 1e-5, False, "silu")
+    xg = x.clone().requires_grad_(True)
+    y = GridnetCudaOp.apply(w, b, r, xg, 33, 8, 1e-5, False, "tanh")  # forward allows it
+    with pytest.raises(RuntimeError, match="cannot backprop through more than 32 inner iterations"):
+        y.sum().backward()
+
+
+def test_gradient_outputs_are_accumulated_into():
+    """The reference adds into the buffers its wrapper zero-fills (gridnet/backend_cuda.py:78-81,
+    src/gridnet_cuda_kernels.cu:424-449); prior contents must survive."""
+    import gridnet_cuda
+
+    shape, bs = (8, 8, 16), 8
+    w, b, r = (t.to(DEV) for t in make_params(shape))
+    x, gy = make_acts(2, shape).to(DEV), make_acts(2, shape, seed=9).to(DEV)
+    outs = [torch.zeros_like(w), torch.zeros_like(b), torch.zeros_like(b), torch.zeros_like(x)]
+    gridnet_cuda.backward(w, b, r, x, gy, *outs, 2, bs, 1e-5, False, "leaky_relu")
+    again = [torch.full_like(t, 0.5) for t in outs]
+    gridnet_cuda.backward(w, b, r, x, gy, *again, 2, bs, 1e-5, False, "leaky_relu")
+    for first, second in zip(outs, again):
+        assert torch.allclose(second, first + 0.5, rtol=1e-5, atol=1e-6)
+
+
+def test_dispatcher_takes_the_hip_path():
+    import warnings
+
+    import gridnet_amd
+
+    shape = (8, 8, 8)
+    w, b, r = (t.to(DEV) for t in make_params(shape))
+    x = make_acts(2, shape).to(DEV)
+    with warnings.catch_warnings():
+        warnings.simplefilter("error")
+        y = gridnet_amd.gridnet_step(w, b, r, x, 2, 8, 1e-5, False, "leaky_relu")
+    ey = gridnet_step_fast(w.cpu().double(), b.cpu().double(), r.cpu().double(), x.cpu().double(),
+                           2, 8, 1e-5, False, "leaky_relu")
+    assert_close(y, ey, what="y")
