@@ -25,9 +25,10 @@ FLAGS = [
 ]
 
 
-def build(verbose: bool = True, extra_flags=()) -> str:
+def build(verbose: bool = True, extra_flags=(), out=None, objdir=None) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    objdir = os.path.join(HERE, "build")
+    objdir = objdir or os.path.join(HERE, "build")
+    out = out or LIB
     os.makedirs(objdir, exist_ok=True)
 
     def compile_one(src):
@@ -48,11 +49,11 @@ def build(verbose: bool = True, extra_flags=()) -> str:
 
     with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as pool:
         objs = list(pool.map(compile_one, SOURCES))
-    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB]
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", out]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.run(cmd, check=True)
-    return LIB
+    return out
 
 
 if __name__ == "__main__":

@@ -1,9 +1,755 @@
-// placeholder, replaced below
+// Tuned fp32 kernels for the block-local update with normalize=false (every configuration the
+// reference's training scripts use: gridnet/scripts/train_mnist.py:51, train_imagenet.py:50).
+//
+// Mapping.  A "slot" is the group of threads that advances ONE (spatial block, batch element)
+// pair: bs*bs*(bs/CPT) threads, each owning CPT consecutive cells of a K-row together with
+// their 27*CPT weights in registers.  A workgroup is NSLOT slots on the same spatial block,
+// each walking its share of the batch elements the workgroup owns, so the 29 parameter planes
+// of a block are fetched once per workgroup and reused for every batch element and every inner
+// iteration.  The (bs+2)^3 window lives in LDS, rows padded to a multiple of 4 floats, so a
+// thread reads the CPT+2 values it needs from each of its 9 neighbour rows with 64/128-bit LDS
+// loads: (CPT+2)*9 loaded values feed 27*CPT FMAs.  Two copies of the window alternate between
+// inner iterations (the frozen halo is written to both), which leaves one barrier per iteration.
+// The next batch element's window is fetched into registers while the current one iterates.
+//
+// Backward, without any atomics (the reference scatters w*delta with shared-memory atomicAdd and
+// adds windows to the grid with global atomicAdd, src/gridnet_cuda_kernels.cu:384-387, 424-449):
+//   * per batch element the inner forward is recomputed, each thread keeping its own x_i and u_i
+//     in a private LDS slab;
+//   * the gradient of an owned cell stays in a register g.  In iteration i each thread writes
+//     delta_i = act'(u_i) g r of its cells into a zero-haloed LDS window and then GATHERS
+//     g += sum_t V[t] * delta_i[c + off_t], where V[t][c] = W[26-t, c + off_t] are the
+//     neighbours' mirrored weights, loaded once per workgroup into registers (zero where the
+//     neighbour lies in another block).  Same shape as the forward stencil, fixed order;
+//   * dW += x_i[nbr] * delta_i accumulates in registers over iterations and batch elements;
+//   * cells of neighbouring blocks (the window's halo) receive sum_t W[t,c'] * delta_i[c'] summed
+//     over i; W does not depend on i, so one pass per batch element over D = sum_i delta_i
+//     suffices.  It runs in gather form from a small LDS table (<= 9 (source, weight) pairs per
+//     halo entry, built once per workgroup) and is written, compacted, to a scratch buffer;
+//   * a second kernel adds each cell's <= 7 halo contributions from its neighbouring blocks to dx
+//     in a fixed order.
+// Parameter gradients leave the kernel once per workgroup: reduced across slots through LDS and,
+// when one workgroup owns the whole batch of its block, written with plain stores.  Results are
+// bitwise reproducible in that case.
+
 #include "common.h"
 #include "launch.h"
+
 namespace gridnet {
-bool step_fast_supports(const StepArgs &, bool) { return false; }
-size_t step_fast_backward_workspace(const StepArgs &) { return 0; }
-int step_forward_fast(const StepArgs &, hipStream_t) { return fail(GRIDNET_ERR_ARGUMENT, "no fast path"); }
-int step_backward_fast(const StepArgs &, hipStream_t) { return fail(GRIDNET_ERR_ARGUMENT, "no fast path"); }
+
+namespace {
+
+template <int BS, int CPT> struct Tile {
+    static constexpr int S = BS + 2;              // window side
+    static constexpr int KT = BS / CPT;           // threads along a K-row
+    static constexpr int TPS = BS * BS * KT;      // threads per slot
+    static constexpr int RS = (S + 3) / 4 * 4;    // LDS row stride (floats)
+    static constexpr int PS = S * RS;             // LDS plane stride
+    static constexpr int WIN = S * PS;            // floats per window copy
+    static constexpr int NWIN = S * S * S;        // window entries
+    static constexpr int NLOAD = (NWIN + TPS - 1) / TPS;  // window entries fetched per thread
+    static constexpr int MID = 4 * S - 4;         // halo entries of a middle plane
+    static constexpr int NH = 2 * S * S + BS * MID;  // halo entries of a window
+    static constexpr int NPAIR = 9;               // (source, weight) pairs per halo entry
+    static_assert(BS % CPT == 0, "cells per thread must divide the block side");
+};
+
+// Compact numbering of the halo: the two full planes i=0 and i=S-1, then for each middle plane
+// the rows j=0 and j=S-1 and the two end cells of every other row.
+template <typename TL>
+__host__ __device__ __forceinline__ void halo_coords(int h, int &wi, int &wj, int &wk) {
+    constexpr int S = TL::S, P = S * S;
+    if (h < 2 * P) {
+        wi = h < P ? 0 : S - 1;
+        const int r = h < P ? h : h - P;
+        wj = r / S;
+        wk = r % S;
+    } else {
+        h -= 2 * P;
+        wi = 1 + h / TL::MID;
+        int r = h % TL::MID;
+        if (r < 2 * S) {
+            wj = r < S ? 0 : S - 1;
+            wk = r < S ? r : r - S;
+        } else {
+            r -= 2 * S;
+            wj = 1 + r / 2;
+            wk = (r & 1) * (S - 1);
+        }
+    }
 }
+
+template <typename TL> __host__ __device__ __forceinline__ int halo_index(int wi, int wj, int wk) {
+    constexpr int S = TL::S, P = S * S;
+    if (wi == 0) return wj * S + wk;
+    if (wi == S - 1) return P + wj * S + wk;
+    const int base = 2 * P + (wi - 1) * TL::MID;
+    if (wj == 0) return base + wk;
+    if (wj == S - 1) return base + S + wk;
+    return base + 2 * S + (wj - 1) * 2 + (wk == S - 1 ? 1 : 0);
+}
+
+// Read CPT+2 consecutive floats starting at an address that is CPT-float aligned.
+template <int CPT> __device__ __forceinline__ void load_row(const float *p, float (&v)[CPT + 2]);
+template <> __device__ __forceinline__ void load_row<1>(const float *p, float (&v)[3]) {
+    v[0] = p[0]; v[1] = p[1]; v[2] = p[2];
+}
+template <> __device__ __forceinline__ void load_row<2>(const float *p, float (&v)[4]) {
+    const float2 a = *reinterpret_cast<const float2 *>(p);
+    const float2 b = *reinterpret_cast<const float2 *>(p + 2);
+    v[0] = a.x; v[1] = a.y; v[2] = b.x; v[3] = b.y;
+}
+template <> __device__ __forceinline__ void load_row<4>(const float *p, float (&v)[6]) {
+    const float4 a = *reinterpret_cast<const float4 *>(p);
+    const float2 b = *reinterpret_cast<const float2 *>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y;
+}
+template <> __device__ __forceinline__ void load_row<8>(const float *p, float (&v)[10]) {
+    const float4 a = *reinterpret_cast<const float4 *>(p);
+    const float4 b = *reinterpret_cast<const float4 *>(p + 4);
+    const float2 c = *reinterpret_cast<const float2 *>(p + 8);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+    v[8] = c.x; v[9] = c.y;
+}
+
+template <int CPT> __device__ __forceinline__ void load_cells(const float *p, float (&v)[CPT]) {
+    if constexpr (CPT == 1) {
+        v[0] = p[0];
+    } else if constexpr (CPT == 2) {
+        const float2 a = *reinterpret_cast<const float2 *>(p);
+        v[0] = a.x; v[1] = a.y;
+    } else {
+#pragma unroll
+        for (int q = 0; q < CPT / 4; ++q) {
+            const float4 a = *reinterpret_cast<const float4 *>(p + 4 * q);
+            v[4 * q] = a.x; v[4 * q + 1] = a.y; v[4 * q + 2] = a.z; v[4 * q + 3] = a.w;
+        }
+    }
+}
+
+template <int CPT> __device__ __forceinline__ void store_cells(float *p, const float (&v)[CPT]) {
+    if constexpr (CPT == 1) {
+        p[0] = v[0];
+    } else if constexpr (CPT == 2) {
+        *reinterpret_cast<float2 *>(p) = make_float2(v[0], v[1]);
+    } else {
+#pragma unroll
+        for (int q = 0; q < CPT / 4; ++q)
+            *reinterpret_cast<float4 *>(p + 4 * q) =
+                make_float4(v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]);
+    }
+}
+
+template <int CPT> __device__ __forceinline__ void add_cells(float *p, const float (&v)[CPT]) {
+    float old[CPT];
+    load_cells<CPT>(p, old);
+#pragma unroll
+    for (int c = 0; c < CPT; ++c) old[c] += v[c];
+    store_cells<CPT>(p, old);
+}
+
+// Where a thread sits: its slot, its cells, and the LDS offsets it uses every iteration.
+template <typename TL, int CPT, int NSLOT> struct Place {
+    int slot, lane;
+    int i, j, kt;         // cell row (i, j) and K-segment within the block
+    int p0, q0, r0;       // block origin in the grid
+    int gc;               // grid index (within a sample) of the first owned cell
+    int row00;            // LDS offset of window row (i, j) at column kt*CPT (tap a = b = 0)
+    int own;              // LDS offset of the first owned cell
+    __device__ __forceinline__ Place(int tid, int blk, int N, int K) {
+        constexpr int bs = TL::S - 2;
+        slot = NSLOT == 1 ? 0 : tid / TL::TPS;
+        lane = tid - slot * TL::TPS;
+        kt = lane % TL::KT;
+        j = (lane / TL::KT) % bs;
+        i = lane / (TL::KT * bs);
+        const int kb = K / bs, nb = N / bs;
+        p0 = (blk / (kb * nb)) * bs;
+        q0 = ((blk / kb) % nb) * bs;
+        r0 = (blk % kb) * bs;
+        gc = ((p0 + i) * N + (q0 + j)) * K + (r0 + kt * CPT);
+        row00 = i * TL::PS + j * TL::RS + kt * CPT;
+        own = row00 + TL::PS + TL::RS + 1;
+    }
+};
+
+// The window entries a thread fetches for every batch element: grid offset within a sample
+// (-1: outside the grid, reads as zero, gridnet/backend_torch.py:63) and LDS offset (-1: none).
+template <typename TL> struct Fetch {
+    int goff[TL::NLOAD];
+    int loff[TL::NLOAD];
+    __device__ __forceinline__ Fetch(int lane, int p0, int q0, int r0, int M, int N, int K) {
+#pragma unroll
+        for (int e = 0; e < TL::NLOAD; ++e) {
+            const int idx = lane + e * TL::TPS;
+            const int wk = idx % TL::S, wj = (idx / TL::S) % TL::S, wi = idx / (TL::S * TL::S);
+            const int gi = p0 + wi - 1, gj = q0 + wj - 1, gk = r0 + wk - 1;
+            const bool in_window = idx < TL::NWIN;
+            const bool in_grid = gi >= 0 && gi < M && gj >= 0 && gj < N && gk >= 0 && gk < K;
+            loff[e] = in_window ? wi * TL::PS + wj * TL::RS + wk : -1;
+            goff[e] = (in_window && in_grid) ? (gi * N + gj) * K + gk : -1;
+        }
+    }
+    __device__ __forceinline__ void fetch(const float *xs, float (&v)[TL::NLOAD]) const {
+#pragma unroll
+        for (int e = 0; e < TL::NLOAD; ++e) v[e] = goff[e] >= 0 ? xs[goff[e]] : 0.f;
+    }
+    // Both window copies receive every entry (the halo must be in both; the block itself is
+    // overwritten by the iterations anyway).
+    __device__ __forceinline__ void commit(float *win, const float (&v)[TL::NLOAD]) const {
+#pragma unroll
+        for (int e = 0; e < TL::NLOAD; ++e)
+            if (loff[e] >= 0) {
+                win[loff[e]] = v[e];
+                win[TL::WIN + loff[e]] = v[e];
+            }
+    }
+};
+
+// u[c] = init[c] + sum over the 27 taps of w[t][c] * window value, taps in raster order.
+template <typename TL, int CPT>
+__device__ __forceinline__ void stencil(const float *win, int row00, const float (&w)[27][CPT],
+                                        const float (&init)[CPT], float (&u)[CPT]) {
+#pragma unroll
+    for (int c = 0; c < CPT; ++c) u[c] = init[c];
+#pragma unroll
+    for (int a = 0; a < 3; ++a)
+#pragma unroll
+        for (int b = 0; b < 3; ++b) {
+            float v[CPT + 2];
+            load_row<CPT>(win + row00 + a * TL::PS + b * TL::RS, v);
+#pragma unroll
+            for (int cc = 0; cc < 3; ++cc)
+#pragma unroll
+                for (int c = 0; c < CPT; ++c) u[c] = fmaf(w[a * 9 + b * 3 + cc][c], v[c + cc], u[c]);
+        }
+}
+
+template <int BS, int CPT, int NSLOT, int ACT>
+__global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_fwd_fast(
+    const float *__restrict__ weight, const float *__restrict__ bias,
+    const float *__restrict__ scale, const float *__restrict__ x, float *__restrict__ y, int B, int M,
+    int N, int K, int inner, int nblk, int nchunk, int chunk_len) {
+    using TL = Tile<BS, CPT>;
+    __shared__ __attribute__((aligned(16))) float lds[NSLOT * 2 * TL::WIN];
+
+    int blk, chunk;
+    split_block_id(blockIdx.x, nblk, nchunk, blk, chunk);
+    const Place<TL, CPT, NSLOT> pl(threadIdx.x, blk, N, K);
+    const Fetch<TL> fx(pl.lane, pl.p0, pl.q0, pl.r0, M, N, K);
+    float *win = lds + pl.slot * (2 * TL::WIN);
+    const long cells = (long)M * N * K;
+
+    float w[27][CPT], bv[CPT], rv[CPT];
+#pragma unroll
+    for (int t = 0; t < 27; ++t) load_cells<CPT>(weight + t * cells + pl.gc, w[t]);
+    load_cells<CPT>(bias + pl.gc, bv);
+    load_cells<CPT>(scale + pl.gc, rv);
+
+    const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
+    float pre[TL::NLOAD];
+    if (s0 + pl.slot < s1) fx.fetch(x + (s0 + pl.slot) * cells, pre);
+    for (int sb = s0; sb < s1; sb += NSLOT) {
+        const int s = sb + pl.slot;
+        const bool active = s < s1;  // a slot past the end idles through the barriers
+        if (active) fx.commit(win, pre);
+        __syncthreads();
+        if (s + NSLOT < s1) fx.fetch(x + (s + NSLOT) * cells, pre);  // next element, in flight
+        float cur[CPT];
+        if (active) {
+#pragma unroll
+            for (int c = 0; c < CPT; ++c) cur[c] = win[pl.own + c];
+        }
+        for (int it = 0; it < inner; ++it) {
+            if (active) {
+                float u[CPT];
+                stencil<TL, CPT>(win + (it & 1) * TL::WIN, pl.row00, w, bv, u);
+#pragma unroll
+                for (int c = 0; c < CPT; ++c) {
+                    cur[c] = fmaf(rv[c], Act<ACT, float>::f(u[c]), cur[c]);
+                    win[((it + 1) & 1) * TL::WIN + pl.own + c] = cur[c];
+                }
+            }
+            __syncthreads();
+        }
+        if (active) store_cells<CPT>(y + s * cells + pl.gc, cur);
+        if (inner == 0) __syncthreads();  // `cur` was read from the window that is rewritten next
+    }
+}
+
+// ---- backward ------------------------------------------------------------------------------
+
+// LDS layout of the backward kernel (floats): per slot [x window x2 | delta window x2 |
+// history: inner slabs of TPS*2*CPT], then one table per workgroup [NH*9 weights | NH*9 offsets].
+template <int BS, int CPT> __host__ __device__ constexpr int bwd_slot_floats(int inner) {
+    return 4 * Tile<BS, CPT>::WIN + inner * Tile<BS, CPT>::TPS * 2 * CPT;
+}
+template <int BS, int CPT, int NSLOT> size_t bwd_lds_bytes(int inner) {
+    using TL = Tile<BS, CPT>;
+    return ((size_t)NSLOT * bwd_slot_floats<BS, CPT>(inner) + 2 * (size_t)TL::NH * TL::NPAIR) *
+           sizeof(float);
+}
+
+template <int BS, int CPT, int NSLOT, int ACT>
+__global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
+    const float *__restrict__ weight, const float *__restrict__ bias,
+    const float *__restrict__ scale, const float *__restrict__ x, const float *__restrict__ dy,
+    float *__restrict__ dweight, float *__restrict__ dbias, float *__restrict__ dscale,
+    float *__restrict__ dx, float *__restrict__ halo_out, int B, int M, int N, int K, int inner,
+    int nblk, int nchunk, int chunk_len, int param_mode, int dx_accumulate) {
+    using TL = Tile<BS, CPT>;
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    constexpr int NT = TL::TPS * NSLOT;
+    const int slot_floats = bwd_slot_floats<BS, CPT>(inner);
+
+    int blk, chunk;
+    split_block_id(blockIdx.x, nblk, nchunk, blk, chunk);
+    const Place<TL, CPT, NSLOT> pl(threadIdx.x, blk, N, K);
+    const Fetch<TL> fx(pl.lane, pl.p0, pl.q0, pl.r0, M, N, K);
+    float *win = lds + pl.slot * slot_floats;
+    float *dwin = win + 2 * TL::WIN;
+    float *hist = dwin + 2 * TL::WIN + pl.lane * CPT;  // + it*TPS*2*CPT (x_i), + TPS*CPT more (u_i)
+    float *tab_w = lds + NSLOT * slot_floats;
+    int *tab_o = reinterpret_cast<int *>(tab_w + TL::NH * TL::NPAIR);
+    const long cells = (long)M * N * K;
+
+    // ---- once per workgroup: parameters, mirrored neighbour weights, halo table ----
+    float w[27][CPT], v[27][CPT], dw[27][CPT], bv[CPT], rv[CPT], db[CPT], dr[CPT];
+#pragma unroll
+    for (int t = 0; t < 27; ++t) {
+        load_cells<CPT>(weight + t * cells + pl.gc, w[t]);
+        // V[t][c] = W[26-t, c + off_t]: what the neighbour at c + off_t multiplies cell c by
+        const int a = t / 9, b = (t / 3) % 3, cc = t % 3;
+        const int ni = pl.i + a - 1, nj = pl.j + b - 1;
+        const bool row_in = ni >= 0 && ni < BS && nj >= 0 && nj < BS;
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) {
+            const int nk = pl.kt * CPT + c + cc - 1;
+            const bool in = row_in && nk >= 0 && nk < BS;
+            v[t][c] = in ? weight[(26 - t) * cells + pl.gc + c + ((a - 1) * N + (b - 1)) * K + (cc - 1)]
+                         : 0.f;
+            dw[t][c] = 0.f;
+        }
+    }
+    load_cells<CPT>(bias + pl.gc, bv);
+    load_cells<CPT>(scale + pl.gc, rv);
+#pragma unroll
+    for (int c = 0; c < CPT; ++c) db[c] = dr[c] = 0.f;
+
+    for (int e = threadIdx.x; e < TL::NH * TL::NPAIR; e += NT) {
+        const int h = e / TL::NPAIR, q = e % TL::NPAIR;
+        int wc[3];
+        halo_coords<TL>(h, wc[0], wc[1], wc[2]);
+        // every axis either pins the source (window face: the adjacent layer of the block) or is
+        // free (source at -1, 0, +1); the free axes consume the two digits of q in order
+        const int digit[2] = {q / 3, q % 3};
+        int used = 0, src[3];
+        bool valid = true;
+#pragma unroll
+        for (int ax = 0; ax < 3; ++ax) {
+            if (wc[ax] == 0) {
+                src[ax] = 1;
+            } else if (wc[ax] == TL::S - 1) {
+                src[ax] = BS;
+            } else {  // a halo entry has at most two free axes
+                src[ax] = wc[ax] + (used == 0 ? digit[0] : digit[1]) - 1;
+                ++used;
+                valid = valid && src[ax] >= 1 && src[ax] <= BS;
+            }
+        }
+        if (used < 2) valid = valid && digit[1] == 1;  // unused digits: keep exactly one copy
+        if (used < 1) valid = valid && digit[0] == 1;
+        float wt = 0.f;
+        int off = 0;
+        if (valid) {
+            // target = source + off_t  =>  tap digits = target - source + 1
+            const int t = (wc[0] - src[0] + 1) * 9 + (wc[1] - src[1] + 1) * 3 + (wc[2] - src[2] + 1);
+            const int gcell = ((pl.p0 + src[0] - 1) * N + (pl.q0 + src[1] - 1)) * K + (pl.r0 + src[2] - 1);
+            wt = weight[t * cells + gcell];
+            off = src[0] * TL::PS + src[1] * TL::RS + src[2];
+        }
+        tab_w[e] = wt;
+        tab_o[e] = off;
+    }
+    // delta windows: the halo stays zero for the whole kernel
+    for (int idx = pl.lane; idx < 2 * TL::WIN; idx += TL::TPS) dwin[idx] = 0.f;
+
+    const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
+    float pre[TL::NLOAD], g[CPT];
+    if (s0 + pl.slot < s1) {
+        fx.fetch(x + (s0 + pl.slot) * cells, pre);
+        load_cells<CPT>(dy + (s0 + pl.slot) * cells + pl.gc, g);
+    }
+    for (int sb = s0; sb < s1; sb += NSLOT) {
+        const int s = sb + pl.slot;
+        const bool active = s < s1;  // a slot past the end idles through the barriers
+        if (active) fx.commit(win, pre);
+        __syncthreads();
+        float gnext[CPT];
+        if (s + NSLOT < s1) {
+            fx.fetch(x + (s + NSLOT) * cells, pre);
+            load_cells<CPT>(dy + (s + NSLOT) * cells + pl.gc, gnext);
+        }
+        float cur[CPT];
+        if (active) {
+#pragma unroll
+            for (int c = 0; c < CPT; ++c) cur[c] = win[pl.own + c];
+        }
+
+        // ---- forward recompute, remembering x_i and u_i of the owned cells ----
+        for (int it = 0; it < inner; ++it) {
+            if (active) {
+                float u[CPT];
+                stencil<TL, CPT>(win + (it & 1) * TL::WIN, pl.row00, w, bv, u);
+                float *h = hist + it * (TL::TPS * 2 * CPT);
+                store_cells<CPT>(h, cur);
+                store_cells<CPT>(h + TL::TPS * CPT, u);
+                if (it + 1 < inner) {  // x_inner itself is never needed
+#pragma unroll
+                    for (int c = 0; c < CPT; ++c) {
+                        cur[c] = fmaf(rv[c], Act<ACT, float>::f(u[c]), cur[c]);
+                        win[((it + 1) & 1) * TL::WIN + pl.own + c] = cur[c];
+                    }
+                }
+            }
+            if (it + 1 < inner) __syncthreads();
+        }
+
+        // ---- reverse sweep: window copy (it & 1) holds x_it, delta copy (it & 1) delta_it ----
+        float dsum[CPT], delta[CPT];
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) dsum[c] = 0.f;
+        for (int it = inner - 1; it >= 0; --it) {
+            if (active) {
+                const float *h = hist + it * (TL::TPS * 2 * CPT);
+                float u[CPT];
+                load_cells<CPT>(h + TL::TPS * CPT, u);
+                if (it + 2 < inner) {  // this copy was overwritten with x_{it+2}: put x_it back
+                    float xi[CPT];
+                    load_cells<CPT>(h, xi);
+#pragma unroll
+                    for (int c = 0; c < CPT; ++c) win[(it & 1) * TL::WIN + pl.own + c] = xi[c];
+                }
+#pragma unroll
+                for (int c = 0; c < CPT; ++c) {
+                    float f, d;
+                    Act<ACT, float>::fd(u[c], f, d);
+                    delta[c] = d * g[c] * rv[c];
+                    dr[c] = fmaf(f, g[c], dr[c]);
+                    db[c] += delta[c];
+                    dsum[c] += delta[c];
+                    dwin[(it & 1) * TL::WIN + pl.own + c] = delta[c];
+                }
+            }
+            __syncthreads();
+            if (active) {
+                const float *xw = win + (it & 1) * TL::WIN + pl.row00;
+                const float *dwn = dwin + (it & 1) * TL::WIN + pl.row00;
+#pragma unroll
+                for (int a = 0; a < 3; ++a)
+#pragma unroll
+                    for (int b = 0; b < 3; ++b) {
+                        float xv[CPT + 2], dv[CPT + 2];
+                        load_row<CPT>(xw + a * TL::PS + b * TL::RS, xv);
+                        load_row<CPT>(dwn + a * TL::PS + b * TL::RS, dv);
+#pragma unroll
+                        for (int cc = 0; cc < 3; ++cc)
+#pragma unroll
+                            for (int c = 0; c < CPT; ++c) {
+                                const int t = a * 9 + b * 3 + cc;
+                                dw[t][c] = fmaf(xv[c + cc], delta[c], dw[t][c]);
+                                g[c] = fmaf(v[t][c], dv[c + cc], g[c]);
+                            }
+                    }
+            }
+        }
+
+        // ---- cells of the neighbouring blocks: one gather pass over D = sum_i delta_i.
+        // Delta copy 1 is free: the last iteration (it = 0) used copy 0, and the readers of
+        // copy 1 (it = 1) are past the barrier of it = 0.
+        if (active) {
+#pragma unroll
+            for (int c = 0; c < CPT; ++c) dwin[TL::WIN + pl.own + c] = dsum[c];
+        }
+        __syncthreads();
+        if (active) {
+            float *hs = halo_out + ((long)s * nblk + blk) * TL::NH;
+            for (int hh = pl.lane; hh < TL::NH; hh += TL::TPS) {
+                float acc = 0.f;
+#pragma unroll
+                for (int q = 0; q < TL::NPAIR; ++q)
+                    acc = fmaf(tab_w[hh * TL::NPAIR + q], dwin[TL::WIN + tab_o[hh * TL::NPAIR + q]], acc);
+                hs[hh] = acc;
+            }
+            if (dx_accumulate) add_cells<CPT>(dx + s * cells + pl.gc, g);
+            else store_cells<CPT>(dx + s * cells + pl.gc, g);
+        }
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) g[c] = gnext[c];
+        // No barrier here: the next commit writes the x windows, whose last readers are past
+        // the barrier above; delta copy 1 is next written after at least one more barrier.
+    }
+
+    // ---- parameter gradients: reduce across slots through LDS, then commit ----
+    if (NSLOT > 1) {
+        __syncthreads();
+        float *red = lds;  // NSLOT * TPS * CPT floats, reused plane by plane
+#pragma unroll
+        for (int t = 0; t < 29; ++t) {
+            float r[CPT];
+#pragma unroll
+            for (int c = 0; c < CPT; ++c) r[c] = t < 27 ? dw[t < 27 ? t : 0][c] : (t == 27 ? db[c] : dr[c]);
+            store_cells<CPT>(red + (pl.slot * TL::TPS + pl.lane) * CPT, r);
+            __syncthreads();
+            if (pl.slot == 0) {
+#pragma unroll
+                for (int q = 1; q < NSLOT; ++q) {
+                    float o[CPT];
+                    load_cells<CPT>(red + (q * TL::TPS + pl.lane) * CPT, o);
+#pragma unroll
+                    for (int c = 0; c < CPT; ++c) r[c] += o[c];
+                }
+#pragma unroll
+                for (int c = 0; c < CPT; ++c) {
+                    if (t < 27) dw[t < 27 ? t : 0][c] = r[c];
+                    else if (t == 27) db[c] = r[c];
+                    else dr[c] = r[c];
+                }
+            }
+            __syncthreads();
+        }
+        if (pl.slot != 0) return;
+    }
+    if (param_mode == kParamStore) {
+#pragma unroll
+        for (int t = 0; t < 27; ++t) store_cells<CPT>(dweight + t * cells + pl.gc, dw[t]);
+        store_cells<CPT>(dbias + pl.gc, db);
+        store_cells<CPT>(dscale + pl.gc, dr);
+    } else if (param_mode == kParamAddExclusive) {
+#pragma unroll
+        for (int t = 0; t < 27; ++t) add_cells<CPT>(dweight + t * cells + pl.gc, dw[t]);
+        add_cells<CPT>(dbias + pl.gc, db);
+        add_cells<CPT>(dscale + pl.gc, dr);
+    } else {
+#pragma unroll
+        for (int t = 0; t < 27; ++t)
+#pragma unroll
+            for (int c = 0; c < CPT; ++c) unsafeAtomicAdd(dweight + t * cells + pl.gc + c, dw[t][c]);
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) {
+            unsafeAtomicAdd(dbias + pl.gc + c, db[c]);
+            unsafeAtomicAdd(dscale + pl.gc + c, dr[c]);
+        }
+    }
+}
+
+// dx[cell] += the halo contributions of the (up to 7) neighbouring blocks whose window
+// contains the cell, in a fixed order.  One thread per cell; cells off every block face skip.
+template <int BS>
+__global__ __launch_bounds__(256) void halo_gather(const float *__restrict__ halo,
+                                                   float *__restrict__ dx, int B, int M, int N, int K,
+                                                   int nblk) {
+    using TL = Tile<BS, 1>;
+    const long cells = (long)M * N * K;
+    const long total = (long)B * cells;
+    const long id = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (id >= total) return;
+    const int s = (int)(id / cells);
+    const int cell = (int)(id - (long)s * cells);
+    const int gk = cell % K, gj = (cell / K) % N, gi = cell / (K * N);
+    const int l[3] = {gi % BS, gj % BS, gk % BS};
+    const int blk3[3] = {gi / BS, gj / BS, gk / BS};
+    const int nb3[3] = {M / BS, N / BS, K / BS};
+    // per axis: the neighbour offsets whose window reaches this cell (0 is the own block)
+    int lo[3], hi[3];
+#pragma unroll
+    for (int ax = 0; ax < 3; ++ax) {
+        lo[ax] = (l[ax] == 0 && blk3[ax] > 0) ? -1 : 0;
+        hi[ax] = (l[ax] == BS - 1 && blk3[ax] < nb3[ax] - 1) ? 1 : 0;
+    }
+    if (lo[0] == 0 && hi[0] == 0 && lo[1] == 0 && hi[1] == 0 && lo[2] == 0 && hi[2] == 0) return;
+    const float *hs = halo + (long)s * nblk * TL::NH;
+    float acc = 0.f;
+    for (int di = lo[0]; di <= hi[0]; ++di)
+        for (int dj = lo[1]; dj <= hi[1]; ++dj)
+            for (int dk = lo[2]; dk <= hi[2]; ++dk) {
+                if (di == 0 && dj == 0 && dk == 0) continue;
+                const int other = ((blk3[0] + di) * nb3[1] + (blk3[1] + dj)) * nb3[2] + (blk3[2] + dk);
+                // this cell in the neighbour's window coordinates
+                const int wi = l[0] + 1 - di * BS, wj = l[1] + 1 - dj * BS, wk = l[2] + 1 - dk * BS;
+                acc += hs[(long)other * TL::NH + halo_index<TL>(wi, wj, wk)];
+            }
+    dx[id] += acc;
+}
+
+__global__ void fill_zero_f32(float *p, long n) {
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long stride = (long)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) p[i] = 0.f;
+}
+
+int fill_zero(float *p, long n, hipStream_t st) {
+    if (n <= 0) return GRIDNET_OK;
+    long blocks = (n + 1023) / 1024;
+    if (blocks > 8192) blocks = 8192;
+    hipLaunchKernelGGL(fill_zero_f32, dim3((unsigned)blocks), dim3(256), 0, st, p, n);
+    return check_launch("fill_zero");
+}
+
+int device_cus() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            cus = n;
+        else
+            cus = 256;
+    }
+    return cus;
+}
+
+struct Plan {
+    int nblk, nchunk, chunk_len;
+};
+
+// The batch is dealt to workgroups in chunks; a chunk is walked NSLOT elements at a time.
+// `resident` = workgroups the chip holds at once: when the blocks alone do not fill it, the
+// batch is split so that the grid is one full wave of workgroups.
+Plan make_plan(const StepArgs &a, int nslot, int resident, bool whole_batch_per_wg) {
+    Plan p;
+    const int bs = a.block_size;
+    p.nblk = (a.M / bs) * (a.N / bs) * (a.K / bs);
+    int nchunk = whole_batch_per_wg ? 1 : resident / p.nblk;
+    const int max_chunks = (a.B + nslot - 1) / nslot;
+    if (nchunk > max_chunks) nchunk = max_chunks;
+    if (nchunk < 1) nchunk = 1;
+    p.chunk_len = (a.B + nchunk - 1) / nchunk;
+    p.chunk_len = (p.chunk_len + nslot - 1) / nslot * nslot;
+    p.nchunk = (a.B + p.chunk_len - 1) / p.chunk_len;
+    return p;
+}
+
+template <int BS, int CPT, int NSLOT, int ACT> int launch_fwd(const StepArgs &a, hipStream_t st) {
+    using TL = Tile<BS, CPT>;
+    auto kern = step_fwd_fast<BS, CPT, NSLOT, ACT>;
+    static int per_cu = 0;
+    if (per_cu == 0) {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, TL::TPS * NSLOT, 0) != hipSuccess ||
+            n < 1)
+            n = 1;
+        per_cu = n;
+    }
+    const Plan p = make_plan(a, NSLOT, per_cu * device_cus(), false);
+    hipLaunchKernelGGL(kern, dim3(p.nblk * p.nchunk), dim3(TL::TPS * NSLOT), 0, st,
+                       (const float *)a.weight, (const float *)a.bias, (const float *)a.scale,
+                       (const float *)a.x, (float *)a.y, a.B, a.M, a.N, a.K, a.inner, p.nblk, p.nchunk,
+                       p.chunk_len);
+    return check_launch("step_fwd_fast");
+}
+
+constexpr size_t kMaxLds = 160 * 1024;
+
+template <int BS, int CPT, int NSLOT, int ACT> int launch_bwd(const StepArgs &a, hipStream_t st) {
+    using TL = Tile<BS, CPT>;
+    const long cells = (long)a.M * a.N * a.K;
+    const size_t lds = bwd_lds_bytes<BS, CPT, NSLOT>(a.inner);
+    auto kern = step_bwd_fast<BS, CPT, NSLOT, ACT>;
+    static bool big_lds_enabled = false;            // per instantiation
+    static int per_cu_cache[kMaxBackwardIters + 1];  // per instantiation, by inner iterations
+    if (lds > 64 * 1024 && !big_lds_enabled) {
+        hipError_t e = hipFuncSetAttribute((const void *)kern,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kMaxLds);
+        if (e != hipSuccess)
+            return fail(GRIDNET_ERR_LAUNCH, "cannot enable %zu bytes of LDS: %s", lds,
+                        hipGetErrorString(e));
+        big_lds_enabled = true;
+    }
+    int &per_cu = per_cu_cache[a.inner];
+    if (per_cu == 0) {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, TL::TPS * NSLOT, lds) != hipSuccess ||
+            n < 1)
+            n = 1;
+        per_cu = n;
+    }
+    const int nblk = (a.M / BS) * (a.N / BS) * (a.K / BS);
+    // one workgroup owns the whole batch of its block (no cross-workgroup reduction of the
+    // parameter gradients) as soon as the blocks alone give every CU a workgroup
+    const bool whole = nblk >= device_cus();
+    const Plan p = make_plan(a, NSLOT, per_cu * device_cus(), whole);
+    const bool new_params = (a.flags & GRIDNET_OVERWRITE_PARAMS) != 0;
+    int param_mode = kParamAtomic;
+    if (p.nchunk == 1) {
+        param_mode = new_params ? kParamStore : kParamAddExclusive;
+    } else if (new_params) {
+        if (int rc = fill_zero((float *)a.dweight, 27 * cells, st)) return rc;
+        if (int rc = fill_zero((float *)a.dbias, cells, st)) return rc;
+        if (int rc = fill_zero((float *)a.dscale, cells, st)) return rc;
+    }
+    const int dx_accumulate = (a.flags & GRIDNET_OVERWRITE_DX) ? 0 : 1;
+    hipLaunchKernelGGL(kern, dim3(p.nblk * p.nchunk), dim3(TL::TPS * NSLOT), lds, st,
+                       (const float *)a.weight, (const float *)a.bias, (const float *)a.scale,
+                       (const float *)a.x, (const float *)a.dy, (float *)a.dweight, (float *)a.dbias,
+                       (float *)a.dscale, (float *)a.dx, (float *)a.workspace, a.B, a.M, a.N, a.K,
+                       a.inner, p.nblk, p.nchunk, p.chunk_len, param_mode, dx_accumulate);
+    if (int rc = check_launch("step_bwd_fast")) return rc;
+    if (nblk > 1) {
+        const long total = (long)a.B * cells;
+        hipLaunchKernelGGL((halo_gather<BS>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                           (const float *)a.workspace, (float *)a.dx, a.B, a.M, a.N, a.K, nblk);
+        if (int rc = check_launch("halo_gather")) return rc;
+    }
+    return GRIDNET_OK;
+}
+
+// ---- the tuned shapes ---------------------------------------------------------------------
+constexpr int kFwdCpt8 = 4, kFwdSlots8 = 1;   // bs=8 forward: 128 threads, 4 cells each
+constexpr int kBwdCpt8 = 2, kBwdSlots8 = 1;   // bs=8 backward: 256 threads, 2 cells each
+constexpr int kFwdCpt4 = 2, kFwdSlots4 = 4;   // bs=4: 32-thread slots, 4 per workgroup
+constexpr int kBwdCpt4 = 2, kBwdSlots4 = 4;
+
+template <bool BWD, int ACT> int dispatch_bs(const StepArgs &a, hipStream_t st) {
+    if (a.block_size == 8) {
+        if (BWD) return launch_bwd<8, kBwdCpt8, kBwdSlots8, ACT>(a, st);
+        return launch_fwd<8, kFwdCpt8, kFwdSlots8, ACT>(a, st);
+    }
+    if (BWD) return launch_bwd<4, kBwdCpt4, kBwdSlots4, ACT>(a, st);
+    return launch_fwd<4, kFwdCpt4, kFwdSlots4, ACT>(a, st);
+}
+
+template <bool BWD> int dispatch(const StepArgs &a, hipStream_t st) {
+    switch (a.activation) {
+        case GRIDNET_ACT_RELU: return dispatch_bs<BWD, GRIDNET_ACT_RELU>(a, st);
+        case GRIDNET_ACT_LEAKY_RELU: return dispatch_bs<BWD, GRIDNET_ACT_LEAKY_RELU>(a, st);
+        case GRIDNET_ACT_SILU: return dispatch_bs<BWD, GRIDNET_ACT_SILU>(a, st);
+        case GRIDNET_ACT_TANH: return dispatch_bs<BWD, GRIDNET_ACT_TANH>(a, st);
+    }
+    return fail(GRIDNET_ERR_ACTIVATION, "unknown activation function: id %d", a.activation);
+}
+
+}  // namespace
+
+bool step_fast_supports(const StepArgs &a, bool backward) {
+    if (a.dtype != GRIDNET_F32 || a.normalize) return false;
+    if (a.block_size != 4 && a.block_size != 8) return false;
+    if (backward) {
+        const size_t lds = a.block_size == 8 ? bwd_lds_bytes<8, kBwdCpt8, kBwdSlots8>(a.inner)
+                                             : bwd_lds_bytes<4, kBwdCpt4, kBwdSlots4>(a.inner);
+        if (lds > kMaxLds) return false;
+    }
+    return true;
+}
+
+size_t step_fast_backward_workspace(const StepArgs &a) {
+    const int bs = a.block_size;
+    const size_t nblk = (size_t)(a.M / bs) * (a.N / bs) * (a.K / bs);
+    const size_t nh = bs == 8 ? Tile<8, 1>::NH : Tile<4, 1>::NH;
+    return (size_t)a.B * nblk * nh * sizeof(float);
+}
+
+int step_forward_fast(const StepArgs &a, hipStream_t st) { return dispatch<false>(a, st); }
+int step_backward_fast(const StepArgs &a, hipStream_t st) { return dispatch<true>(a, st); }
+
+}  // namespace gridnet

@@ -12,7 +12,8 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libgridnet_hip.so")
+# GRIDNET_HIP_LIBRARY lets a caller point at another build of the same ABI
+LIB_PATH = os.environ.get("GRIDNET_HIP_LIBRARY") or os.path.join(_HERE, "libgridnet_hip.so")
 
 F32, F64 = 0, 1
 OVERWRITE_PARAMS = 1
