@@ -21,7 +21,11 @@
 //     g += sum_t V[t] * delta_i[c + off_t], where V[t][c] = W[26-t, c + off_t] are the
 //     neighbours' mirrored weights, loaded once per workgroup into registers (zero where the
 //     neighbour lies in another block).  Same shape as the forward stencil, fixed order;
-//   * dW += x_i[nbr] * delta_i accumulates in registers over iterations and batch elements;
+//   * the same delta rows give the weight gradients: x_i[c] * delta_i[c + off_t] is the gradient
+//     of the NEIGHBOUR's mirrored weight W[26-t, c + off_t], and this thread is the only one that
+//     ever contributes to it, so it accumulates in a register over iterations and batch elements
+//     (the x window is not re-read in the reverse sweep).  Weights whose tap reads a halo entry
+//     see a frozen x there: their gradient is x_halo * sum_i delta_i, one pass per batch element;
 //   * cells of neighbouring blocks (the window's halo) receive sum_t W[t,c'] * delta_i[c'] summed
 //     over i; W does not depend on i, so one pass per batch element over D = sum_i delta_i
 //     suffices.  It runs in gather form from a small LDS table (<= 9 (source, weight) pairs per
@@ -87,6 +91,22 @@ template <typename TL> __host__ __device__ __forceinline__ int halo_index(int wi
     if (wj == 0) return base + wk;
     if (wj == S - 1) return base + S + wk;
     return base + 2 * S + (wj - 1) * 2 + (wk == S - 1 ? 1 : 0);
+}
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every global
+// load in flight, which would stall each inner iteration on the prefetch of the next batch
+// element; global memory needs no ordering inside these kernels.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// Wait for every global load issued so far (s_waitcnt vmcnt(0) only).  Placed once after the
+// per-workgroup parameter loads: with those known complete, the waits the compiler inserts
+// inside the batch loop no longer cover the prefetch of the next batch element as well.
+__device__ __forceinline__ void wait_global_loads() {
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt = 0, expcnt = 7, lgkmcnt = 15 (gfx9 encoding)
 }
 
 // Read CPT+2 consecutive floats starting at an address that is CPT-float aligned.
@@ -160,9 +180,11 @@ template <typename TL, int CPT, int NSLOT> struct Place {
         constexpr int bs = TL::S - 2;
         slot = NSLOT == 1 ? 0 : tid / TL::TPS;
         lane = tid - slot * TL::TPS;
+        // kt fastest, then i, then j: the lanes an LDS access serves together then differ in
+        // the plane index, and the plane stride (S*RS = 120 or 48 floats) spreads them over banks
         kt = lane % TL::KT;
-        j = (lane / TL::KT) % bs;
-        i = lane / (TL::KT * bs);
+        i = (lane / TL::KT) % bs;
+        j = lane / (TL::KT * bs);
         const int kb = K / bs, nb = N / bs;
         p0 = (blk / (kb * nb)) * bs;
         q0 = ((blk / kb) % nb) * bs;
@@ -245,6 +267,7 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_fwd_fast(
     for (int t = 0; t < 27; ++t) load_cells<CPT>(weight + t * cells + pl.gc, w[t]);
     load_cells<CPT>(bias + pl.gc, bv);
     load_cells<CPT>(scale + pl.gc, rv);
+    wait_global_loads();
 
     const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
     float pre[TL::NLOAD];
@@ -253,7 +276,7 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_fwd_fast(
         const int s = sb + pl.slot;
         const bool active = s < s1;  // a slot past the end idles through the barriers
         if (active) fx.commit(win, pre);
-        __syncthreads();
+        lds_barrier();
         if (s + NSLOT < s1) fx.fetch(x + (s + NSLOT) * cells, pre);  // next element, in flight
         float cur[CPT];
         if (active) {
@@ -270,10 +293,10 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_fwd_fast(
                     win[((it + 1) & 1) * TL::WIN + pl.own + c] = cur[c];
                 }
             }
-            __syncthreads();
+            lds_barrier();
         }
         if (active) store_cells<CPT>(y + s * cells + pl.gc, cur);
-        if (inner == 0) __syncthreads();  // `cur` was read from the window that is rewritten next
+        if (inner == 0) lds_barrier();  // `cur` was read from the window that is rewritten next
     }
 }
 
@@ -290,6 +313,42 @@ template <int BS, int CPT, int NSLOT> size_t bwd_lds_bytes(int inner) {
            sizeof(float);
 }
 
+// Pair q (0..8) of halo entry h: the block cell `src` (window coordinates) whose tap `t` reads
+// that halo entry.  Every window axis either pins the source (entry on a window face: the
+// adjacent layer of the block) or is free (source at -1, 0, +1 along it); the free axes consume
+// the two base-3 digits of q in order, unused digits must be 1 so each pair appears once.
+template <typename TL, int BS>
+__device__ __forceinline__ bool halo_pair(int h, int q, int &t, int (&src)[3]) {
+    int wc[3];
+    halo_coords<TL>(h, wc[0], wc[1], wc[2]);
+    const int d0 = q / 3, d1 = q % 3;
+    int used = 0;
+    bool valid = true;
+#pragma unroll
+    for (int ax = 0; ax < 3; ++ax) {
+        if (wc[ax] == 0) {
+            src[ax] = 1;
+        } else if (wc[ax] == TL::S - 1) {
+            src[ax] = BS;
+        } else {  // a halo entry has at most two free axes
+            src[ax] = wc[ax] + (used == 0 ? d0 : d1) - 1;
+            ++used;
+            valid = valid && src[ax] >= 1 && src[ax] <= BS;
+        }
+    }
+    if (used < 2) valid = valid && d1 == 1;
+    if (used < 1) valid = valid && d0 == 1;
+    // halo entry = source + off_t  =>  tap digits = entry - source + 1
+    t = (wc[0] - src[0] + 1) * 9 + (wc[1] - src[1] + 1) * 3 + (wc[2] - src[2] + 1);
+    return valid;
+}
+
+__device__ __forceinline__ void commit_grad(float *p, float v, int mode) {
+    if (mode == kParamStore) *p = v;
+    else if (mode == kParamAddExclusive) *p += v;
+    else unsafeAtomicAdd(p, v);
+}
+
 template <int BS, int CPT, int NSLOT, int ACT>
 __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
     const float *__restrict__ weight, const float *__restrict__ bias,
@@ -300,6 +359,7 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
     using TL = Tile<BS, CPT>;
     extern __shared__ __attribute__((aligned(16))) float lds[];
     constexpr int NT = TL::TPS * NSLOT;
+    constexpr int NHPT = (TL::NH + TL::TPS - 1) / TL::TPS;  // halo entries per thread
     const int slot_floats = bwd_slot_floats<BS, CPT>(inner);
 
     int blk, chunk;
@@ -314,11 +374,14 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
     const long cells = (long)M * N * K;
 
     // ---- once per workgroup: parameters, mirrored neighbour weights, halo table ----
-    float w[27][CPT], v[27][CPT], dw[27][CPT], bv[CPT], rv[CPT], db[CPT], dr[CPT];
+    // w : this cell's weights (forward recompute)
+    // v : V[t][c] = W[26-t, c + off_t], what the neighbour at c + off_t multiplies cell c by
+    // nw: gradient of that same neighbour weight; it is the product of this cell's x and the
+    //     neighbour's delta summed over iterations and batch, so this thread owns it completely
+    float w[27][CPT], v[27][CPT], nw[27][CPT], bv[CPT], rv[CPT], db[CPT], dr[CPT];
 #pragma unroll
     for (int t = 0; t < 27; ++t) {
         load_cells<CPT>(weight + t * cells + pl.gc, w[t]);
-        // V[t][c] = W[26-t, c + off_t]: what the neighbour at c + off_t multiplies cell c by
         const int a = t / 9, b = (t / 3) % 3, cc = t % 3;
         const int ni = pl.i + a - 1, nj = pl.j + b - 1;
         const bool row_in = ni >= 0 && ni < BS && nj >= 0 && nj < BS;
@@ -328,7 +391,7 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
             const bool in = row_in && nk >= 0 && nk < BS;
             v[t][c] = in ? weight[(26 - t) * cells + pl.gc + c + ((a - 1) * N + (b - 1)) * K + (cc - 1)]
                          : 0.f;
-            dw[t][c] = 0.f;
+            nw[t][c] = 0.f;
         }
     }
     load_cells<CPT>(bias + pl.gc, bv);
@@ -337,33 +400,11 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
     for (int c = 0; c < CPT; ++c) db[c] = dr[c] = 0.f;
 
     for (int e = threadIdx.x; e < TL::NH * TL::NPAIR; e += NT) {
-        const int h = e / TL::NPAIR, q = e % TL::NPAIR;
-        int wc[3];
-        halo_coords<TL>(h, wc[0], wc[1], wc[2]);
-        // every axis either pins the source (window face: the adjacent layer of the block) or is
-        // free (source at -1, 0, +1); the free axes consume the two digits of q in order
-        const int digit[2] = {q / 3, q % 3};
-        int used = 0, src[3];
-        bool valid = true;
-#pragma unroll
-        for (int ax = 0; ax < 3; ++ax) {
-            if (wc[ax] == 0) {
-                src[ax] = 1;
-            } else if (wc[ax] == TL::S - 1) {
-                src[ax] = BS;
-            } else {  // a halo entry has at most two free axes
-                src[ax] = wc[ax] + (used == 0 ? digit[0] : digit[1]) - 1;
-                ++used;
-                valid = valid && src[ax] >= 1 && src[ax] <= BS;
-            }
-        }
-        if (used < 2) valid = valid && digit[1] == 1;  // unused digits: keep exactly one copy
-        if (used < 1) valid = valid && digit[0] == 1;
+        int t, src[3];
+        const bool valid = halo_pair<TL, BS>(e / TL::NPAIR, e % TL::NPAIR, t, src);
         float wt = 0.f;
-        int off = 0;
+        int off = 0;  // invalid pairs read window entry 0, a halo corner of the delta window: zero
         if (valid) {
-            // target = source + off_t  =>  tap digits = target - source + 1
-            const int t = (wc[0] - src[0] + 1) * 9 + (wc[1] - src[1] + 1) * 3 + (wc[2] - src[2] + 1);
             const int gcell = ((pl.p0 + src[0] - 1) * N + (pl.q0 + src[1] - 1)) * K + (pl.r0 + src[2] - 1);
             wt = weight[t * cells + gcell];
             off = src[0] * TL::PS + src[1] * TL::RS + src[2];
@@ -371,8 +412,22 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
         tab_w[e] = wt;
         tab_o[e] = off;
     }
+    // the halo entries this thread serves for every batch element, and the gradients of the
+    // weights whose tap reads them: x on the halo is frozen, so these need only D = sum_i delta_i
+    int hoff[NHPT];
+    float hw[NHPT][TL::NPAIR];
+#pragma unroll
+    for (int k = 0; k < NHPT; ++k) {
+        const int hh = pl.lane + k * TL::TPS;
+        int wi = 0, wj = 0, wk = 0;
+        if (hh < TL::NH) halo_coords<TL>(hh, wi, wj, wk);
+        hoff[k] = wi * TL::PS + wj * TL::RS + wk;
+#pragma unroll
+        for (int q = 0; q < TL::NPAIR; ++q) hw[k][q] = 0.f;
+    }
     // delta windows: the halo stays zero for the whole kernel
     for (int idx = pl.lane; idx < 2 * TL::WIN; idx += TL::TPS) dwin[idx] = 0.f;
+    wait_global_loads();
 
     const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
     float pre[TL::NLOAD], g[CPT];
@@ -384,7 +439,7 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
         const int s = sb + pl.slot;
         const bool active = s < s1;  // a slot past the end idles through the barriers
         if (active) fx.commit(win, pre);
-        __syncthreads();
+        lds_barrier();
         float gnext[CPT];
         if (s + NSLOT < s1) {
             fx.fetch(x + (s + NSLOT) * cells, pre);
@@ -412,52 +467,45 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
                     }
                 }
             }
-            if (it + 1 < inner) __syncthreads();
+            if (it + 1 < inner) lds_barrier();
         }
 
-        // ---- reverse sweep: window copy (it & 1) holds x_it, delta copy (it & 1) delta_it ----
-        float dsum[CPT], delta[CPT];
+        // ---- reverse sweep: delta window copy (it & 1) holds delta_it ----
+        float dsum[CPT], xi[CPT];
 #pragma unroll
         for (int c = 0; c < CPT; ++c) dsum[c] = 0.f;
         for (int it = inner - 1; it >= 0; --it) {
             if (active) {
                 const float *h = hist + it * (TL::TPS * 2 * CPT);
                 float u[CPT];
+                load_cells<CPT>(h, xi);
                 load_cells<CPT>(h + TL::TPS * CPT, u);
-                if (it + 2 < inner) {  // this copy was overwritten with x_{it+2}: put x_it back
-                    float xi[CPT];
-                    load_cells<CPT>(h, xi);
-#pragma unroll
-                    for (int c = 0; c < CPT; ++c) win[(it & 1) * TL::WIN + pl.own + c] = xi[c];
-                }
 #pragma unroll
                 for (int c = 0; c < CPT; ++c) {
                     float f, d;
                     Act<ACT, float>::fd(u[c], f, d);
-                    delta[c] = d * g[c] * rv[c];
+                    const float delta = d * g[c] * rv[c];
                     dr[c] = fmaf(f, g[c], dr[c]);
-                    db[c] += delta[c];
-                    dsum[c] += delta[c];
-                    dwin[(it & 1) * TL::WIN + pl.own + c] = delta[c];
+                    db[c] += delta;
+                    dsum[c] += delta;
+                    dwin[(it & 1) * TL::WIN + pl.own + c] = delta;
                 }
             }
-            __syncthreads();
+            lds_barrier();
             if (active) {
-                const float *xw = win + (it & 1) * TL::WIN + pl.row00;
                 const float *dwn = dwin + (it & 1) * TL::WIN + pl.row00;
 #pragma unroll
                 for (int a = 0; a < 3; ++a)
 #pragma unroll
                     for (int b = 0; b < 3; ++b) {
-                        float xv[CPT + 2], dv[CPT + 2];
-                        load_row<CPT>(xw + a * TL::PS + b * TL::RS, xv);
+                        float dv[CPT + 2];
                         load_row<CPT>(dwn + a * TL::PS + b * TL::RS, dv);
 #pragma unroll
                         for (int cc = 0; cc < 3; ++cc)
 #pragma unroll
                             for (int c = 0; c < CPT; ++c) {
                                 const int t = a * 9 + b * 3 + cc;
-                                dw[t][c] = fmaf(xv[c + cc], delta[c], dw[t][c]);
+                                nw[t][c] = fmaf(xi[c], dv[c + cc], nw[t][c]);
                                 g[c] = fmaf(v[t][c], dv[c + cc], g[c]);
                             }
                     }
@@ -467,79 +515,99 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
         // ---- cells of the neighbouring blocks: one gather pass over D = sum_i delta_i.
         // Delta copy 1 is free: the last iteration (it = 0) used copy 0, and the readers of
         // copy 1 (it = 1) are past the barrier of it = 0.
+        float xh[NHPT];
         if (active) {
 #pragma unroll
             for (int c = 0; c < CPT; ++c) dwin[TL::WIN + pl.own + c] = dsum[c];
+            // x on the halo (identical in both window copies), read before the barrier so that
+            // the next element's window may be committed right after it
+#pragma unroll
+            for (int k = 0; k < NHPT; ++k) xh[k] = win[hoff[k]];
         }
-        __syncthreads();
+        lds_barrier();
         if (active) {
             float *hs = halo_out + ((long)s * nblk + blk) * TL::NH;
-            for (int hh = pl.lane; hh < TL::NH; hh += TL::TPS) {
-                float acc = 0.f;
 #pragma unroll
-                for (int q = 0; q < TL::NPAIR; ++q)
-                    acc = fmaf(tab_w[hh * TL::NPAIR + q], dwin[TL::WIN + tab_o[hh * TL::NPAIR + q]], acc);
-                hs[hh] = acc;
+            for (int k = 0; k < NHPT; ++k) {
+                const int hh = pl.lane + k * TL::TPS;
+                if (hh < TL::NH) {
+                    float acc = 0.f;
+#pragma unroll
+                    for (int q = 0; q < TL::NPAIR; ++q) {
+                        const float d = dwin[TL::WIN + tab_o[hh * TL::NPAIR + q]];
+                        acc = fmaf(tab_w[hh * TL::NPAIR + q], d, acc);
+                        hw[k][q] = fmaf(xh[k], d, hw[k][q]);
+                    }
+                    hs[hh] = acc;
+                }
             }
             if (dx_accumulate) add_cells<CPT>(dx + s * cells + pl.gc, g);
             else store_cells<CPT>(dx + s * cells + pl.gc, g);
         }
 #pragma unroll
         for (int c = 0; c < CPT; ++c) g[c] = gnext[c];
-        // No barrier here: the next commit writes the x windows, whose last readers are past
-        // the barrier above; delta copy 1 is next written after at least one more barrier.
+        // No barrier here: the next commit writes only the x windows, whose last readers are
+        // before the barrier above; delta copy 1 is next written after at least one more barrier.
     }
 
     // ---- parameter gradients: reduce across slots through LDS, then commit ----
     if (NSLOT > 1) {
-        __syncthreads();
-        float *red = lds;  // NSLOT * TPS * CPT floats, reused plane by plane
-#pragma unroll
-        for (int t = 0; t < 29; ++t) {
-            float r[CPT];
-#pragma unroll
-            for (int c = 0; c < CPT; ++c) r[c] = t < 27 ? dw[t < 27 ? t : 0][c] : (t == 27 ? db[c] : dr[c]);
-            store_cells<CPT>(red + (pl.slot * TL::TPS + pl.lane) * CPT, r);
-            __syncthreads();
+        float *red = lds;  // NSLOT * TPS floats, reused value by value
+        auto reduce = [&](float &val) {
+            lds_barrier();
+            red[pl.slot * TL::TPS + pl.lane] = val;
+            lds_barrier();
             if (pl.slot == 0) {
 #pragma unroll
-                for (int q = 1; q < NSLOT; ++q) {
-                    float o[CPT];
-                    load_cells<CPT>(red + (q * TL::TPS + pl.lane) * CPT, o);
-#pragma unroll
-                    for (int c = 0; c < CPT; ++c) r[c] += o[c];
-                }
-#pragma unroll
-                for (int c = 0; c < CPT; ++c) {
-                    if (t < 27) dw[t < 27 ? t : 0][c] = r[c];
-                    else if (t == 27) db[c] = r[c];
-                    else dr[c] = r[c];
-                }
+                for (int q = 1; q < NSLOT; ++q) val += red[q * TL::TPS + pl.lane];
             }
-            __syncthreads();
-        }
-        if (pl.slot != 0) return;
-    }
-    if (param_mode == kParamStore) {
-#pragma unroll
-        for (int t = 0; t < 27; ++t) store_cells<CPT>(dweight + t * cells + pl.gc, dw[t]);
-        store_cells<CPT>(dbias + pl.gc, db);
-        store_cells<CPT>(dscale + pl.gc, dr);
-    } else if (param_mode == kParamAddExclusive) {
-#pragma unroll
-        for (int t = 0; t < 27; ++t) add_cells<CPT>(dweight + t * cells + pl.gc, dw[t]);
-        add_cells<CPT>(dbias + pl.gc, db);
-        add_cells<CPT>(dscale + pl.gc, dr);
-    } else {
+        };
 #pragma unroll
         for (int t = 0; t < 27; ++t)
 #pragma unroll
-            for (int c = 0; c < CPT; ++c) unsafeAtomicAdd(dweight + t * cells + pl.gc + c, dw[t][c]);
+            for (int c = 0; c < CPT; ++c) reduce(nw[t][c]);
 #pragma unroll
         for (int c = 0; c < CPT; ++c) {
-            unsafeAtomicAdd(dbias + pl.gc + c, db[c]);
-            unsafeAtomicAdd(dscale + pl.gc + c, dr[c]);
+            reduce(db[c]);
+            reduce(dr[c]);
         }
+#pragma unroll
+        for (int k = 0; k < NHPT; ++k)
+#pragma unroll
+            for (int q = 0; q < TL::NPAIR; ++q) reduce(hw[k][q]);
+        if (pl.slot != 0) return;
+    }
+#pragma unroll
+    for (int t = 0; t < 27; ++t) {
+        const int a = t / 9, b = (t / 3) % 3, cc = t % 3;
+        const int ni = pl.i + a - 1, nj = pl.j + b - 1;
+        const bool row_in = ni >= 0 && ni < BS && nj >= 0 && nj < BS;
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) {
+            const int nk = pl.kt * CPT + c + cc - 1;
+            if (row_in && nk >= 0 && nk < BS)
+                commit_grad(dweight + (26 - t) * cells + pl.gc + c + ((a - 1) * N + (b - 1)) * K + (cc - 1),
+                            nw[t][c], param_mode);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < NHPT; ++k) {
+        const int hh = pl.lane + k * TL::TPS;
+        if (hh < TL::NH) {
+#pragma unroll
+            for (int q = 0; q < TL::NPAIR; ++q) {
+                int t, src[3];
+                if (halo_pair<TL, BS>(hh, q, t, src)) {
+                    const int gcell = ((pl.p0 + src[0] - 1) * N + (pl.q0 + src[1] - 1)) * K + (pl.r0 + src[2] - 1);
+                    commit_grad(dweight + t * cells + gcell, hw[k][q], param_mode);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < CPT; ++c) {
+        commit_grad(dbias + pl.gc + c, db[c], param_mode);
+        commit_grad(dscale + pl.gc + c, dr[c], param_mode);
     }
 }
 
