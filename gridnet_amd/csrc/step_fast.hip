@@ -228,23 +228,55 @@ template <typename TL> struct Fetch {
     }
 };
 
+// Visit the 9 neighbour rows of a thread in tap order with the LDS reads running DEPTH rows
+// ahead of the arithmetic: row r + DEPTH is requested before row r is consumed, and scheduling
+// barriers keep the compiler from collapsing that order when registers are tight (it otherwise
+// falls back to load, wait, 12 FMAs, load, ... and every row pays the full LDS latency).
+template <typename TL, int CPT, int DEPTH, typename F>
+__device__ __forceinline__ void for_each_row(const float *rows, F &&consume) {
+    float buf[DEPTH][CPT + 2];
+#pragma unroll
+    for (int r = 0; r < DEPTH && r < 9; ++r)
+        load_row<CPT>(rows + (r / 3) * TL::PS + (r % 3) * TL::RS, buf[r]);
+#pragma unroll
+    for (int r = 0; r < 9; ++r) {
+        __builtin_amdgcn_sched_barrier(0);
+        consume(r, buf[r % DEPTH]);
+        if (r + DEPTH < 9) {
+            __builtin_amdgcn_sched_barrier(0);
+            load_row<CPT>(rows + ((r + DEPTH) / 3) * TL::PS + ((r + DEPTH) % 3) * TL::RS, buf[r % DEPTH]);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+}
+
 // u[c] = init[c] + sum over the 27 taps of w[t][c] * window value, taps in raster order.
-template <typename TL, int CPT>
+template <typename TL, int CPT, int DEPTH = 9>
 __device__ __forceinline__ void stencil(const float *win, int row00, const float (&w)[27][CPT],
                                         const float (&init)[CPT], float (&u)[CPT]) {
 #pragma unroll
     for (int c = 0; c < CPT; ++c) u[c] = init[c];
+    if constexpr (DEPTH >= 9) {  // all rows requested up front; the compiler orders the rest
 #pragma unroll
-    for (int a = 0; a < 3; ++a)
+        for (int a = 0; a < 3; ++a)
 #pragma unroll
-        for (int b = 0; b < 3; ++b) {
-            float v[CPT + 2];
-            load_row<CPT>(win + row00 + a * TL::PS + b * TL::RS, v);
+            for (int b = 0; b < 3; ++b) {
+                float v[CPT + 2];
+                load_row<CPT>(win + row00 + a * TL::PS + b * TL::RS, v);
+#pragma unroll
+                for (int cc = 0; cc < 3; ++cc)
+#pragma unroll
+                    for (int c = 0; c < CPT; ++c)
+                        u[c] = fmaf(w[a * 9 + b * 3 + cc][c], v[c + cc], u[c]);
+            }
+    } else {
+        for_each_row<TL, CPT, DEPTH>(win + row00, [&](int r, const float (&v)[CPT + 2]) {
 #pragma unroll
             for (int cc = 0; cc < 3; ++cc)
 #pragma unroll
-                for (int c = 0; c < CPT; ++c) u[c] = fmaf(w[a * 9 + b * 3 + cc][c], v[c + cc], u[c]);
-        }
+                for (int c = 0; c < CPT; ++c) u[c] = fmaf(w[r * 3 + cc][c], v[c + cc], u[c]);
+        });
+    }
 }
 
 template <int BS, int CPT, int NSLOT, int ACT>
@@ -301,6 +333,10 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_fwd_fast(
 }
 
 // ---- backward ------------------------------------------------------------------------------
+#ifndef EXP_BWD_DEPTH
+#define EXP_BWD_DEPTH 4
+#endif
+constexpr int kBwdDepth = EXP_BWD_DEPTH;  // neighbour rows requested ahead of the arithmetic
 
 // LDS layout of the backward kernel (floats): per slot [x window x2 | delta window x2 |
 // history: inner slabs of TPS*2*CPT], then one table per workgroup [NH*9 weights | NH*9 offsets].
@@ -455,7 +491,7 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
         for (int it = 0; it < inner; ++it) {
             if (active) {
                 float u[CPT];
-                stencil<TL, CPT>(win + (it & 1) * TL::WIN, pl.row00, w, bv, u);
+                stencil<TL, CPT, kBwdDepth>(win + (it & 1) * TL::WIN, pl.row00, w, bv, u);
                 float *h = hist + it * (TL::TPS * 2 * CPT);
                 store_cells<CPT>(h, cur);
                 store_cells<CPT>(h + TL::TPS * CPT, u);
@@ -494,21 +530,15 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
             lds_barrier();
             if (active) {
                 const float *dwn = dwin + (it & 1) * TL::WIN + pl.row00;
+                for_each_row<TL, CPT, kBwdDepth>(dwn, [&](int r, const float (&dv)[CPT + 2]) {
 #pragma unroll
-                for (int a = 0; a < 3; ++a)
+                    for (int cc = 0; cc < 3; ++cc)
 #pragma unroll
-                    for (int b = 0; b < 3; ++b) {
-                        float dv[CPT + 2];
-                        load_row<CPT>(dwn + a * TL::PS + b * TL::RS, dv);
-#pragma unroll
-                        for (int cc = 0; cc < 3; ++cc)
-#pragma unroll
-                            for (int c = 0; c < CPT; ++c) {
-                                const int t = a * 9 + b * 3 + cc;
-                                nw[t][c] = fmaf(xi[c], dv[c + cc], nw[t][c]);
-                                g[c] = fmaf(v[t][c], dv[c + cc], g[c]);
-                            }
-                    }
+                        for (int c = 0; c < CPT; ++c) {
+                            nw[r * 3 + cc][c] = fmaf(xi[c], dv[c + cc], nw[r * 3 + cc][c]);
+                            g[c] = fmaf(v[r * 3 + cc][c], dv[c + cc], g[c]);
+                        }
+                });
             }
         }
 
