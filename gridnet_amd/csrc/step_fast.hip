@@ -641,43 +641,49 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
     }
 }
 
-// dx[cell] += the halo contributions of the (up to 7) neighbouring blocks whose window
-// contains the cell, in a fixed order.  One thread per cell; cells off every block face skip.
+// dx[cell] += the halo contributions of the (up to 7) neighbouring blocks whose window contains
+// the cell, added in a fixed order.  One thread owns one K-row of one block (bs cells): whether
+// a neighbour in i or j reaches the row is decided once per row, and those contributions are
+// bs consecutive floats of the neighbour's compacted halo; only the two end cells of the row
+// also see neighbours in k.  blockIdx.y = sample.
 template <int BS>
 __global__ __launch_bounds__(256) void halo_gather(const float *__restrict__ halo,
-                                                   float *__restrict__ dx, int B, int M, int N, int K,
-                                                   int nblk) {
+                                                   float *__restrict__ dx, int M, int N, int K,
+                                                   int nblk, int rows_per_sample) {
     using TL = Tile<BS, 1>;
-    const long cells = (long)M * N * K;
-    const long total = (long)B * cells;
-    const long id = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (id >= total) return;
-    const int s = (int)(id / cells);
-    const int cell = (int)(id - (long)s * cells);
-    const int gk = cell % K, gj = (cell / K) % N, gi = cell / (K * N);
-    const int l[3] = {gi % BS, gj % BS, gk % BS};
-    const int blk3[3] = {gi / BS, gj / BS, gk / BS};
-    const int nb3[3] = {M / BS, N / BS, K / BS};
-    // per axis: the neighbour offsets whose window reaches this cell (0 is the own block)
-    int lo[3], hi[3];
+    const int row = blockIdx.x * blockDim.x + threadIdx.x;  // (gi, gj, bk), bk fastest
+    if (row >= rows_per_sample) return;
+    const int kb = K / BS, nb = N / BS, mb = M / BS;
+    const int bk = row % kb;
+    const int gj = (row / kb) % N;
+    const int gi = row / (kb * N);
+    const int li = gi % BS, lj = gj % BS, bi = gi / BS, bj = gj / BS;
+    const int di_lo = (li == 0 && bi > 0) ? -1 : 0, di_hi = (li == BS - 1 && bi < mb - 1) ? 1 : 0;
+    const int dj_lo = (lj == 0 && bj > 0) ? -1 : 0, dj_hi = (lj == BS - 1 && bj < nb - 1) ? 1 : 0;
+    const float *hs = halo + (size_t)blockIdx.y * nblk * TL::NH;
+    float acc[BS];
 #pragma unroll
-    for (int ax = 0; ax < 3; ++ax) {
-        lo[ax] = (l[ax] == 0 && blk3[ax] > 0) ? -1 : 0;
-        hi[ax] = (l[ax] == BS - 1 && blk3[ax] < nb3[ax] - 1) ? 1 : 0;
-    }
-    if (lo[0] == 0 && hi[0] == 0 && lo[1] == 0 && hi[1] == 0 && lo[2] == 0 && hi[2] == 0) return;
-    const float *hs = halo + (long)s * nblk * TL::NH;
-    float acc = 0.f;
-    for (int di = lo[0]; di <= hi[0]; ++di)
-        for (int dj = lo[1]; dj <= hi[1]; ++dj)
-            for (int dk = lo[2]; dk <= hi[2]; ++dk) {
-                if (di == 0 && dj == 0 && dk == 0) continue;
-                const int other = ((blk3[0] + di) * nb3[1] + (blk3[1] + dj)) * nb3[2] + (blk3[2] + dk);
-                // this cell in the neighbour's window coordinates
-                const int wi = l[0] + 1 - di * BS, wj = l[1] + 1 - dj * BS, wk = l[2] + 1 - dk * BS;
-                acc += hs[(long)other * TL::NH + halo_index<TL>(wi, wj, wk)];
+    for (int c = 0; c < BS; ++c) acc[c] = 0.f;
+    for (int di = di_lo; di <= di_hi; ++di)
+        for (int dj = dj_lo; dj <= dj_hi; ++dj) {
+            const int wi = li + 1 - di * BS, wj = lj + 1 - dj * BS;  // row in the neighbour's window
+            const int other = ((bi + di) * nb + (bj + dj)) * kb + bk;
+            if (di != 0 || dj != 0) {  // the neighbour's halo holds the whole row, contiguously
+                const float *src = hs + (size_t)other * TL::NH + halo_index<TL>(wi, wj, 1);
+#pragma unroll
+                for (int c = 0; c < BS; ++c) acc[c] += src[c];
             }
-    dx[id] += acc;
+            // neighbours one block further along k reach only the row's end cells
+            if (bk > 0) acc[0] += hs[(size_t)(other - 1) * TL::NH + halo_index<TL>(wi, wj, BS + 1)];
+            if (bk < kb - 1) acc[BS - 1] += hs[(size_t)(other + 1) * TL::NH + halo_index<TL>(wi, wj, 0)];
+        }
+    float *out = dx + ((size_t)blockIdx.y * M * N + (size_t)gi * N + gj) * K + bk * BS;
+#pragma unroll
+    for (int q = 0; q < BS / 4; ++q) {
+        float4 o = *reinterpret_cast<float4 *>(out + 4 * q);
+        o.x += acc[4 * q]; o.y += acc[4 * q + 1]; o.z += acc[4 * q + 2]; o.w += acc[4 * q + 3];
+        *reinterpret_cast<float4 *>(out + 4 * q) = o;
+    }
 }
 
 __global__ void fill_zero_f32(float *p, long n) {
@@ -794,9 +800,9 @@ template <int BS, int CPT, int NSLOT, int ACT> int launch_bwd(const StepArgs &a,
                        a.inner, p.nblk, p.nchunk, p.chunk_len, param_mode, dx_accumulate);
     if (int rc = check_launch("step_bwd_fast")) return rc;
     if (nblk > 1) {
-        const long total = (long)a.B * cells;
-        hipLaunchKernelGGL((halo_gather<BS>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
-                           (const float *)a.workspace, (float *)a.dx, a.B, a.M, a.N, a.K, nblk);
+        const int rows = a.M * a.N * (a.K / BS);
+        hipLaunchKernelGGL((halo_gather<BS>), dim3((rows + 255) / 256, a.B), dim3(256), 0, st,
+                           (const float *)a.workspace, (float *)a.dx, a.M, a.N, a.K, nblk, rows);
         if (int rc = check_launch("halo_gather")) return rc;
     }
     return GRIDNET_OK;
