@@ -97,6 +97,9 @@ template <typename TL> __host__ __device__ __forceinline__ int halo_index(int wi
 // load in flight, which would stall each inner iteration on the prefetch of the next batch
 // element; global memory needs no ordering inside these kernels.
 __device__ __forceinline__ void lds_barrier() {
+#ifdef EXP_NOBARRIER
+    return;
+#endif
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
@@ -195,35 +198,72 @@ template <typename TL, int CPT, int NSLOT> struct Place {
     }
 };
 
-// The window entries a thread fetches for every batch element: grid offset within a sample
-// (-1: outside the grid, reads as zero, gridnet/backend_torch.py:63) and LDS offset (-1: none).
+// Fetching a window: one thread per window row (S*S rows of S entries; the first S*S threads
+// of a slot take one row each, or several when the slot is small).  The bs cells of the block
+// that lie in a row are contiguous and 16-byte aligned in the grid, so they come in as float4;
+// the two end entries belong to the neighbouring blocks (or lie outside the grid and read as
+// zero, gridnet/backend_torch.py:63).
 template <typename TL> struct Fetch {
-    int goff[TL::NLOAD];
-    int loff[TL::NLOAD];
+    static constexpr int S = TL::S, BS = TL::S - 2;
+    static constexpr int NROW = S * S;
+    static constexpr int RPT = (NROW + TL::TPS - 1) / TL::TPS;  // rows per thread
+    int goff[RPT];   // grid offset (within a sample) of the row's first block cell; off-grid rows
+                     // point at a valid address and are zeroed when committed
+    int loff[RPT];   // LDS offset of the row's first entry, -1: no row for this thread
+    bool ok[RPT];    // the row lies inside the grid
+    int lo_d, hi_d;  // address deltas of the two end entries (0 when they are off-grid)
+    bool lo_ok, hi_ok;
     __device__ __forceinline__ Fetch(int lane, int p0, int q0, int r0, int M, int N, int K) {
+        lo_ok = r0 > 0;
+        hi_ok = r0 + BS < K;
+        lo_d = lo_ok ? -1 : 0;
+        hi_d = hi_ok ? BS : 0;
 #pragma unroll
-        for (int e = 0; e < TL::NLOAD; ++e) {
-            const int idx = lane + e * TL::TPS;
-            const int wk = idx % TL::S, wj = (idx / TL::S) % TL::S, wi = idx / (TL::S * TL::S);
-            const int gi = p0 + wi - 1, gj = q0 + wj - 1, gk = r0 + wk - 1;
-            const bool in_window = idx < TL::NWIN;
-            const bool in_grid = gi >= 0 && gi < M && gj >= 0 && gj < N && gk >= 0 && gk < K;
-            loff[e] = in_window ? wi * TL::PS + wj * TL::RS + wk : -1;
-            goff[e] = (in_window && in_grid) ? (gi * N + gj) * K + gk : -1;
+        for (int e = 0; e < RPT; ++e) {
+            const int row = lane + e * TL::TPS;
+            const int wj = row % S, wi = row / S;
+            const int gi = p0 + wi - 1, gj = q0 + wj - 1;
+            const bool have = row < NROW;
+            ok[e] = have && gi >= 0 && gi < M && gj >= 0 && gj < N;
+            loff[e] = have ? wi * TL::PS + wj * TL::RS : -1;
+            // rows outside the grid (and threads without a row) read row (0, 0) of the sample at
+            // the block's own columns: always in bounds, also for the two end entries, because
+            // lo_d / hi_d are non-zero only when columns r0-1 / r0+bs exist
+            goff[e] = ok[e] ? (gi * N + gj) * K + r0 : r0;
         }
     }
-    __device__ __forceinline__ void fetch(const float *xs, float (&v)[TL::NLOAD]) const {
+    // Unconditional loads (no branches, no register initialisation in front of them).
+    __device__ __forceinline__ void fetch(const float *xs, float (&v)[RPT][S]) const {
 #pragma unroll
-        for (int e = 0; e < TL::NLOAD; ++e) v[e] = goff[e] >= 0 ? xs[goff[e]] : 0.f;
+        for (int e = 0; e < RPT; ++e) {
+            const float *p = xs + goff[e];
+#pragma unroll
+            for (int q = 0; q < BS / 4; ++q) {
+                const float4 t = *reinterpret_cast<const float4 *>(p + 4 * q);
+                v[e][1 + 4 * q] = t.x; v[e][2 + 4 * q] = t.y; v[e][3 + 4 * q] = t.z; v[e][4 + 4 * q] = t.w;
+            }
+            v[e][0] = p[lo_d];
+            v[e][S - 1] = p[hi_d];
+        }
     }
     // Both window copies receive every entry (the halo must be in both; the block itself is
-    // overwritten by the iterations anyway).
-    __device__ __forceinline__ void commit(float *win, const float (&v)[TL::NLOAD]) const {
+    // overwritten by the iterations anyway).  Row starts are 8-byte aligned.
+    __device__ __forceinline__ void commit(float *win, const float (&v)[RPT][S]) const {
 #pragma unroll
-        for (int e = 0; e < TL::NLOAD; ++e)
+        for (int e = 0; e < RPT; ++e)
             if (loff[e] >= 0) {
-                win[loff[e]] = v[e];
-                win[TL::WIN + loff[e]] = v[e];
+                float r[S];
+#pragma unroll
+                for (int q = 0; q < S; ++q) r[q] = ok[e] ? v[e][q] : 0.f;
+                if (!lo_ok) r[0] = 0.f;
+                if (!hi_ok) r[S - 1] = 0.f;
+#pragma unroll
+                for (int copy = 0; copy < 2; ++copy) {
+                    float *row = win + copy * TL::WIN + loff[e];
+#pragma unroll
+                    for (int q = 0; q < S / 2; ++q)
+                        *reinterpret_cast<float2 *>(row + 2 * q) = make_float2(r[2 * q], r[2 * q + 1]);
+                }
             }
     }
 };
@@ -262,12 +302,22 @@ __device__ __forceinline__ void stencil(const float *win, int row00, const float
 #pragma unroll
             for (int b = 0; b < 3; ++b) {
                 float v[CPT + 2];
+#ifdef EXP_NOLOAD
+#pragma unroll
+                for (int q = 0; q < CPT + 2; ++q) v[q] = init[q % CPT] + (float)(a + b);
+#else
                 load_row<CPT>(win + row00 + a * TL::PS + b * TL::RS, v);
+#endif
+#ifdef EXP_NOFMA
+#pragma unroll
+                for (int q = 0; q < CPT + 2; ++q) u[q % CPT] += v[q];
+#else
 #pragma unroll
                 for (int cc = 0; cc < 3; ++cc)
 #pragma unroll
                     for (int c = 0; c < CPT; ++c)
                         u[c] = fmaf(w[a * 9 + b * 3 + cc][c], v[c + cc], u[c]);
+#endif
             }
     } else {
         for_each_row<TL, CPT, DEPTH>(win + row00, [&](int r, const float (&v)[CPT + 2]) {
@@ -278,6 +328,11 @@ __device__ __forceinline__ void stencil(const float *win, int row00, const float
         });
     }
 }
+
+#ifndef EXP_FWD_DEPTH
+#define EXP_FWD_DEPTH 9
+#endif
+constexpr int kFwdDepth = EXP_FWD_DEPTH;  // neighbour rows requested ahead of the arithmetic
 
 template <int BS, int CPT, int NSLOT, int ACT>
 __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_fwd_fast(
@@ -302,13 +357,19 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_fwd_fast(
     wait_global_loads();
 
     const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
-    float pre[TL::NLOAD];
+    float pre[Fetch<TL>::RPT][TL::S];
     if (s0 + pl.slot < s1) fx.fetch(x + (s0 + pl.slot) * cells, pre);
+    // The result of an element is stored one element late, after the next window has been
+    // committed: the wait for the prefetched window would otherwise also wait for a store that
+    // was issued an instant earlier (loads and stores share one in-order counter).
+    float done[CPT];
+    int done_s = -1;
     for (int sb = s0; sb < s1; sb += NSLOT) {
         const int s = sb + pl.slot;
         const bool active = s < s1;  // a slot past the end idles through the barriers
         if (active) fx.commit(win, pre);
         lds_barrier();
+        if (done_s >= 0) store_cells<CPT>(y + done_s * cells + pl.gc, done);
         if (s + NSLOT < s1) fx.fetch(x + (s + NSLOT) * cells, pre);  // next element, in flight
         float cur[CPT];
         if (active) {
@@ -318,7 +379,7 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_fwd_fast(
         for (int it = 0; it < inner; ++it) {
             if (active) {
                 float u[CPT];
-                stencil<TL, CPT>(win + (it & 1) * TL::WIN, pl.row00, w, bv, u);
+                stencil<TL, CPT, kFwdDepth>(win + (it & 1) * TL::WIN, pl.row00, w, bv, u);
 #pragma unroll
                 for (int c = 0; c < CPT; ++c) {
                     cur[c] = fmaf(rv[c], Act<ACT, float>::f(u[c]), cur[c]);
@@ -327,9 +388,12 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_fwd_fast(
             }
             lds_barrier();
         }
-        if (active) store_cells<CPT>(y + s * cells + pl.gc, cur);
+        done_s = active ? s : -1;
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) done[c] = cur[c];
         if (inner == 0) lds_barrier();  // `cur` was read from the window that is rewritten next
     }
+    if (done_s >= 0) store_cells<CPT>(y + done_s * cells + pl.gc, done);
 }
 
 // ---- backward ------------------------------------------------------------------------------
@@ -466,7 +530,7 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
     wait_global_loads();
 
     const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
-    float pre[TL::NLOAD], g[CPT];
+    float pre[Fetch<TL>::RPT][TL::S], g[CPT];
     if (s0 + pl.slot < s1) {
         fx.fetch(x + (s0 + pl.slot) * cells, pre);
         load_cells<CPT>(dy + (s0 + pl.slot) * cells + pl.gc, g);
