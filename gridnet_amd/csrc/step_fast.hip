@@ -109,7 +109,9 @@ __device__ __forceinline__ void lds_barrier() {
 // per-workgroup parameter loads: with those known complete, the waits the compiler inserts
 // inside the batch loop no longer cover the prefetch of the next batch element as well.
 __device__ __forceinline__ void wait_global_loads() {
+    __builtin_amdgcn_sched_barrier(0);   // keep the loads above and the loop below where they are
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt = 0, expcnt = 7, lgkmcnt = 15 (gfx9 encoding)
+    __builtin_amdgcn_sched_barrier(0);
 }
 
 // Read CPT+2 consecutive floats starting at an address that is CPT-float aligned.
