@@ -93,24 +93,22 @@ template <typename T> __device__ __forceinline__ T block_sum(T v, T *scratch, in
     return total;
 }
 
-// Workgroup id -> (spatial block, batch chunk) so that the workgroups that share a spatial
-// block -- and therefore its 29 parameter planes -- land on the same XCD (ids are dealt to
-// the 8 XCDs round-robin) and hit that XCD's L2 instead of refetching.
-__device__ __forceinline__ void split_block_id(int wg, int nblk, int nchunk, int &blk, int &chunk) {
-    constexpr int X = 8;
-    const int groups = nblk / X;  // full groups of 8 spatial blocks
-    const int per_group = X * nchunk;
-    const int grp = wg / per_group;
-    if (grp < groups) {
-        const int r = wg - grp * per_group;
-        blk = grp * X + (r % X);
-        chunk = r / X;
-    } else {  // ragged tail: plain chunk-minor order
-        const int r = wg - groups * per_group;
-        const int tail = nblk - groups * X;
-        blk = groups * X + (r % tail);
-        chunk = r / tail;
-    }
+// Workgroup id -> (spatial block, batch chunk).  Workgroup ids are dealt to the 8 XCDs
+// round-robin and every XCD has its own L2, so XCD x is given a CONTIGUOUS range of spatial
+// blocks (raster order: neighbours along K, then N): neighbouring blocks share halo cells and
+// whole cache lines of every K-row, and the chunks of one block share its 29 parameter planes.
+// Handing neighbouring blocks to different XCDs makes each L2 fetch those lines again.
+// The grid is padded to 8 * ceil(nblk / 8) * nchunk workgroups; returns false for the padding.
+constexpr int kXcds = 8;
+__host__ __device__ __forceinline__ int padded_grid(int nblk, int nchunk) {
+    return kXcds * ((nblk + kXcds - 1) / kXcds) * nchunk;
+}
+__device__ __forceinline__ bool split_block_id(int wg, int nblk, int nchunk, int &blk, int &chunk) {
+    const int per_xcd = (nblk + kXcds - 1) / kXcds;
+    const int xcd = wg % kXcds, slot = wg / kXcds;
+    blk = xcd * per_xcd + slot / nchunk;
+    chunk = slot % nchunk;
+    return slot / nchunk < per_xcd && blk < nblk;
 }
 
 }  // namespace gridnet

@@ -345,7 +345,7 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_fwd_fast(
     __shared__ __attribute__((aligned(16))) float lds[NSLOT * 2 * TL::WIN];
 
     int blk, chunk;
-    split_block_id(blockIdx.x, nblk, nchunk, blk, chunk);
+    if (!split_block_id(blockIdx.x, nblk, nchunk, blk, chunk)) return;  // grid padding
     const Place<TL, CPT, NSLOT> pl(threadIdx.x, blk, N, K);
     const Fetch<TL> fx(pl.lane, pl.p0, pl.q0, pl.r0, M, N, K);
     float *win = lds + pl.slot * (2 * TL::WIN);
@@ -465,7 +465,7 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
     const int slot_floats = bwd_slot_floats<BS, CPT>(inner);
 
     int blk, chunk;
-    split_block_id(blockIdx.x, nblk, nchunk, blk, chunk);
+    if (!split_block_id(blockIdx.x, nblk, nchunk, blk, chunk)) return;  // grid padding
     const Place<TL, CPT, NSLOT> pl(threadIdx.x, blk, N, K);
     const Fetch<TL> fx(pl.lane, pl.p0, pl.q0, pl.r0, M, N, K);
     float *win = lds + pl.slot * slot_floats;
@@ -812,7 +812,7 @@ template <int BS, int CPT, int NSLOT, int ACT> int launch_fwd(const StepArgs &a,
         per_cu = n;
     }
     const Plan p = make_plan(a, NSLOT, per_cu * device_cus(), false);
-    hipLaunchKernelGGL(kern, dim3(p.nblk * p.nchunk), dim3(TL::TPS * NSLOT), 0, st,
+    hipLaunchKernelGGL(kern, dim3(padded_grid(p.nblk, p.nchunk)), dim3(TL::TPS * NSLOT), 0, st,
                        (const float *)a.weight, (const float *)a.bias, (const float *)a.scale,
                        (const float *)a.x, (float *)a.y, a.B, a.M, a.N, a.K, a.inner, p.nblk, p.nchunk,
                        p.chunk_len);
@@ -859,7 +859,7 @@ template <int BS, int CPT, int NSLOT, int ACT> int launch_bwd(const StepArgs &a,
         if (int rc = fill_zero((float *)a.dscale, cells, st)) return rc;
     }
     const int dx_accumulate = (a.flags & GRIDNET_OVERWRITE_DX) ? 0 : 1;
-    hipLaunchKernelGGL(kern, dim3(p.nblk * p.nchunk), dim3(TL::TPS * NSLOT), lds, st,
+    hipLaunchKernelGGL(kern, dim3(padded_grid(p.nblk, p.nchunk)), dim3(TL::TPS * NSLOT), lds, st,
                        (const float *)a.weight, (const float *)a.bias, (const float *)a.scale,
                        (const float *)a.x, (const float *)a.dy, (float *)a.dweight, (float *)a.dbias,
                        (float *)a.dscale, (float *)a.dx, (float *)a.workspace, a.B, a.M, a.N, a.K,

@@ -84,7 +84,7 @@ __global__ __launch_bounds__(BS *BS *BS) void step_fwd_generic(
 
     const int tid = threadIdx.x;
     int blk, chunk;
-    split_block_id(blockIdx.x, nblk, nchunk, blk, chunk);
+    if (!split_block_id(blockIdx.x, nblk, nchunk, blk, chunk)) return;  // grid padding
     const int kb = K / BS, nb = N / BS;
     const int p0 = (blk / (kb * nb)) * BS, q0 = ((blk / kb) % nb) * BS, r0 = (blk % kb) * BS;
     const int ci = tid / (BS * BS), cj = (tid / BS) % BS, ck = tid % BS;
@@ -131,7 +131,7 @@ __global__ __launch_bounds__(BS *BS *BS) void step_bwd_generic(
 
     const int tid = threadIdx.x;
     int blk, chunk;
-    split_block_id(blockIdx.x, nblk, nchunk, blk, chunk);
+    if (!split_block_id(blockIdx.x, nblk, nchunk, blk, chunk)) return;  // grid padding
     const int kb = K / BS, nb = N / BS;
     const int p0 = (blk / (kb * nb)) * BS, q0 = ((blk / kb) % nb) * BS, r0 = (blk % kb) * BS;
     const int ci = tid / (BS * BS), cj = (tid / BS) % BS, ck = tid % BS;
@@ -254,7 +254,7 @@ template <typename T> __global__ void fill_zero_kernel(T *p, long n) {
 
 template <typename T, int BS, int ACT>
 int launch_fwd_norm(const StepArgs &a, int nblk, int nchunk, int chunk_len, hipStream_t st) {
-    dim3 grid(nblk * nchunk), block(Geo<BS>::NT);
+    dim3 grid(padded_grid(nblk, nchunk)), block(Geo<BS>::NT);
     auto args = [&](auto kern) {
         hipLaunchKernelGGL(kern, grid, block, 0, st, (const T *)a.weight, (const T *)a.bias,
                            (const T *)a.scale, (const T *)a.x, (T *)a.y, a.B, a.M, a.N, a.K,
@@ -268,7 +268,7 @@ int launch_fwd_norm(const StepArgs &a, int nblk, int nchunk, int chunk_len, hipS
 template <typename T, int BS, int ACT>
 int launch_bwd_norm(const StepArgs &a, int nblk, int nchunk, int chunk_len, int param_mode,
                     hipStream_t st) {
-    dim3 grid(nblk * nchunk), block(Geo<BS>::NT);
+    dim3 grid(padded_grid(nblk, nchunk)), block(Geo<BS>::NT);
     auto args = [&](auto kern) {
         hipLaunchKernelGGL(kern, grid, block, 0, st, (const T *)a.weight, (const T *)a.bias,
                            (const T *)a.scale, (const T *)a.x, (const T *)a.dy, (T *)a.dweight,
