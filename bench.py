@@ -132,6 +132,14 @@ def main():
     wall, kernel_s = gpu_run(wl, args.steps, args.warmup)
     bytes_ = wl.algorithmic_bytes()
     dominant = max(kernel_s, key=lambda k: kernel_s[k])
+    # HBM bytes per call of that entry point, from the committed rocprofv3 --pmc summary
+    # (FETCH_SIZE and WRITE_SIZE runs, scaled by a copy kernel of known size); null if absent
+    traffic = None
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as fh:
+            traffic = json.load(fh).get(args.workload, {}).get(dominant)
+    except OSError:
+        pass
     dom_s = kernel_s[dominant]
     achieved = bytes_[dominant] / dom_s / 1e9
     out = {
@@ -158,7 +166,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None,
+            "traffic": traffic,
         },
     }
     if not args.no_cpu_baseline:
