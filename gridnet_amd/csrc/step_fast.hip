@@ -445,6 +445,33 @@ __device__ __forceinline__ bool halo_pair(int h, int q, int &t, int (&src)[3]) {
     return valid;
 }
 
+// The decode of every (halo entry, pair) is the same for all workgroups and all calls: it is
+// evaluated once per process into a device table, one word per pair:
+// bit 31 = valid, bits 16..20 = tap, bits 0..15 = LDS offset of the source cell in a window.
+__device__ int g_pair_words8[Tile<8, 1>::NH * Tile<8, 1>::NPAIR];
+__device__ int g_pair_words4[Tile<4, 1>::NH * Tile<4, 1>::NPAIR];
+template <int BS> __device__ __forceinline__ int *pair_words() {
+    if constexpr (BS == 8) return g_pair_words8;
+    else return g_pair_words4;
+}
+template <int BS> __global__ void build_pair_words() {
+    using TL = Tile<BS, 1>;
+    const int e = blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= TL::NH * TL::NPAIR) return;
+    int t, src[3];
+    const bool valid = halo_pair<TL, BS>(e / TL::NPAIR, e % TL::NPAIR, t, src);
+    pair_words<BS>()[e] = valid ? (int)(0x80000000u | (unsigned)(t << 16) |
+                                        (unsigned)(src[0] * TL::PS + src[1] * TL::RS + src[2]))
+                                : 0;
+}
+// Grid index (within a sample) of the source cell of a pair word, for a block at (p0, q0, r0).
+template <typename TL>
+__device__ __forceinline__ int pair_source_cell(int word, int p0, int q0, int r0, int N, int K) {
+    const int off = word & 0xffff;
+    const int s0 = off / TL::PS, s1 = (off % TL::PS) / TL::RS, s2 = off % TL::RS;
+    return ((p0 + s0 - 1) * N + (q0 + s1 - 1)) * K + (r0 + s2 - 1);
+}
+
 __device__ __forceinline__ void commit_grad(float *p, float v, int mode) {
     if (mode == kParamStore) *p = v;
     else if (mode == kParamAddExclusive) *p += v;
@@ -471,8 +498,8 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
     float *win = lds + pl.slot * slot_floats;
     float *dwin = win + 2 * TL::WIN;
     float *hist = dwin + 2 * TL::WIN + pl.lane * CPT;  // + it*TPS*2*CPT (x_i), + TPS*CPT more (u_i)
-    float *tab_w = lds + NSLOT * slot_floats;
-    int *tab_o = reinterpret_cast<int *>(tab_w + TL::NH * TL::NPAIR);
+    // per workgroup: (weight, source offset) of every pair, 8 bytes each
+    float2 *tab = reinterpret_cast<float2 *>(lds + NSLOT * slot_floats);
     const long cells = (long)M * N * K;
 
     // ---- once per workgroup: parameters, mirrored neighbour weights, halo table ----
@@ -501,18 +528,27 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
 #pragma unroll
     for (int c = 0; c < CPT; ++c) db[c] = dr[c] = 0.f;
 
-    for (int e = threadIdx.x; e < TL::NH * TL::NPAIR; e += NT) {
-        int t, src[3];
-        const bool valid = halo_pair<TL, BS>(e / TL::NPAIR, e % TL::NPAIR, t, src);
-        float wt = 0.f;
-        int off = 0;  // invalid pairs read window entry 0, a halo corner of the delta window: zero
-        if (valid) {
-            const int gcell = ((pl.p0 + src[0] - 1) * N + (pl.q0 + src[1] - 1)) * K + (pl.r0 + src[2] - 1);
-            wt = weight[t * cells + gcell];
-            off = src[0] * TL::PS + src[1] * TL::RS + src[2];
+    {
+        constexpr int NP = TL::NH * TL::NPAIR, NE = (NP + NT - 1) / NT;
+        const int *words = pair_words<BS>();
+        int word[NE];
+        float wt[NE];
+#pragma unroll
+        for (int n = 0; n < NE; ++n) {
+            const int e = threadIdx.x + n * NT;
+            word[n] = e < NP ? words[e] : 0;
         }
-        tab_w[e] = wt;
-        tab_o[e] = off;
+#pragma unroll
+        for (int n = 0; n < NE; ++n)  // all gathers in flight together
+            wt[n] = word[n] < 0 ? weight[((word[n] >> 16) & 31) * cells +
+                                         pair_source_cell<TL>(word[n], pl.p0, pl.q0, pl.r0, N, K)]
+                                : 0.f;
+#pragma unroll
+        for (int n = 0; n < NE; ++n) {
+            const int e = threadIdx.x + n * NT;
+            // invalid pairs read window entry 0, a halo corner of the delta window: zero
+            if (e < NP) tab[e] = make_float2(wt[n], __int_as_float(word[n] & 0xffff));
+        }
     }
     // the halo entries this thread serves for every batch element, and the gradients of the
     // weights whose tap reads them: x on the halo is frozen, so these need only D = sum_i delta_i
@@ -627,11 +663,14 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
             for (int k = 0; k < NHPT; ++k) {
                 const int hh = pl.lane + k * TL::TPS;
                 if (hh < TL::NH) {
+                    float2 ent[TL::NPAIR];
+#pragma unroll
+                    for (int q = 0; q < TL::NPAIR; ++q) ent[q] = tab[hh * TL::NPAIR + q];
                     float acc = 0.f;
 #pragma unroll
                     for (int q = 0; q < TL::NPAIR; ++q) {
-                        const float d = dwin[TL::WIN + tab_o[hh * TL::NPAIR + q]];
-                        acc = fmaf(tab_w[hh * TL::NPAIR + q], d, acc);
+                        const float d = dwin[TL::WIN + __float_as_int(ent[q].y)];
+                        acc = fmaf(ent[q].x, d, acc);
                         hw[k][q] = fmaf(xh[k], d, hw[k][q]);
                     }
                     hs[hh] = acc;
@@ -692,11 +731,11 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
         if (hh < TL::NH) {
 #pragma unroll
             for (int q = 0; q < TL::NPAIR; ++q) {
-                int t, src[3];
-                if (halo_pair<TL, BS>(hh, q, t, src)) {
-                    const int gcell = ((pl.p0 + src[0] - 1) * N + (pl.q0 + src[1] - 1)) * K + (pl.r0 + src[2] - 1);
-                    commit_grad(dweight + t * cells + gcell, hw[k][q], param_mode);
-                }
+                const int word = pair_words<BS>()[hh * TL::NPAIR + q];
+                if (word < 0)
+                    commit_grad(dweight + ((word >> 16) & 31) * cells +
+                                    pair_source_cell<TL>(word, pl.p0, pl.q0, pl.r0, N, K),
+                                hw[k][q], param_mode);
             }
         }
     }
@@ -859,6 +898,17 @@ template <int BS, int CPT, int NSLOT, int ACT> int launch_bwd(const StepArgs &a,
         if (int rc = fill_zero((float *)a.dscale, cells, st)) return rc;
     }
     const int dx_accumulate = (a.flags & GRIDNET_OVERWRITE_DX) ? 0 : 1;
+    {   // the pair table of this block size, once per device (idempotent, stream-ordered)
+        static bool built[64] = {false};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess) dev = -1;
+        if (dev >= 0 && dev < 64 && !built[dev]) {
+            constexpr int NP = Tile<BS, 1>::NH * Tile<BS, 1>::NPAIR;
+            hipLaunchKernelGGL((build_pair_words<BS>), dim3((NP + 255) / 256), dim3(256), 0, st);
+            if (int rc = check_launch("build_pair_words")) return rc;
+            built[dev] = true;
+        }
+    }
     hipLaunchKernelGGL(kern, dim3(padded_grid(p.nblk, p.nchunk)), dim3(TL::TPS * NSLOT), lds, st,
                        (const float *)a.weight, (const float *)a.bias, (const float *)a.scale,
                        (const float *)a.x, (const float *)a.dy, (float *)a.dweight, (float *)a.dbias,
