@@ -97,9 +97,6 @@ template <typename TL> __host__ __device__ __forceinline__ int halo_index(int wi
 // load in flight, which would stall each inner iteration on the prefetch of the next batch
 // element; global memory needs no ordering inside these kernels.
 __device__ __forceinline__ void lds_barrier() {
-#ifdef EXP_NOBARRIER
-    return;
-#endif
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
@@ -304,22 +301,12 @@ __device__ __forceinline__ void stencil(const float *win, int row00, const float
 #pragma unroll
             for (int b = 0; b < 3; ++b) {
                 float v[CPT + 2];
-#ifdef EXP_NOLOAD
-#pragma unroll
-                for (int q = 0; q < CPT + 2; ++q) v[q] = init[q % CPT] + (float)(a + b);
-#else
                 load_row<CPT>(win + row00 + a * TL::PS + b * TL::RS, v);
-#endif
-#ifdef EXP_NOFMA
-#pragma unroll
-                for (int q = 0; q < CPT + 2; ++q) u[q % CPT] += v[q];
-#else
 #pragma unroll
                 for (int cc = 0; cc < 3; ++cc)
 #pragma unroll
                     for (int c = 0; c < CPT; ++c)
                         u[c] = fmaf(w[a * 9 + b * 3 + cc][c], v[c + cc], u[c]);
-#endif
             }
     } else {
         for_each_row<TL, CPT, DEPTH>(win + row00, [&](int r, const float (&v)[CPT + 2]) {
@@ -331,10 +318,7 @@ __device__ __forceinline__ void stencil(const float *win, int row00, const float
     }
 }
 
-#ifndef EXP_FWD_DEPTH
-#define EXP_FWD_DEPTH 9
-#endif
-constexpr int kFwdDepth = EXP_FWD_DEPTH;  // neighbour rows requested ahead of the arithmetic
+constexpr int kFwdDepth = 9;  // neighbour rows requested ahead of the arithmetic
 
 template <int BS, int CPT, int NSLOT, int ACT>
 __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_fwd_fast(
@@ -399,10 +383,7 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_fwd_fast(
 }
 
 // ---- backward ------------------------------------------------------------------------------
-#ifndef EXP_BWD_DEPTH
-#define EXP_BWD_DEPTH 4
-#endif
-constexpr int kBwdDepth = EXP_BWD_DEPTH;  // neighbour rows requested ahead of the arithmetic
+constexpr int kBwdDepth = 4;  // neighbour rows requested ahead of the arithmetic
 
 // LDS layout of the backward kernel (floats): per slot [x window x2 | delta window x2 |
 // history: inner slabs of TPS*2*CPT], then one table per workgroup [NH*9 weights | NH*9 offsets].
@@ -573,11 +554,27 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
         fx.fetch(x + (s0 + pl.slot) * cells, pre);
         load_cells<CPT>(dy + (s0 + pl.slot) * cells + pl.gc, g);
     }
+    // The gradients of an element leave one element late, after the next window has been
+    // committed: the wait for the prefetched window would otherwise also wait for stores that
+    // were issued an instant earlier (loads and stores share one in-order counter).
+    float g_done[CPT], h_done[NHPT];
+    int done_s = -1;
+    auto flush_done = [&]() {
+        if (done_s < 0) return;
+        float *hs = halo_out + ((long)done_s * nblk + blk) * TL::NH;
+#pragma unroll
+        for (int k = 0; k < NHPT; ++k)
+            if (pl.lane + k * TL::TPS < TL::NH) hs[pl.lane + k * TL::TPS] = h_done[k];
+        if (dx_accumulate) add_cells<CPT>(dx + done_s * cells + pl.gc, g_done);
+        else store_cells<CPT>(dx + done_s * cells + pl.gc, g_done);
+        done_s = -1;
+    };
     for (int sb = s0; sb < s1; sb += NSLOT) {
         const int s = sb + pl.slot;
         const bool active = s < s1;  // a slot past the end idles through the barriers
         if (active) fx.commit(win, pre);
         lds_barrier();
+        flush_done();
         float gnext[CPT];
         if (s + NSLOT < s1) {
             fx.fetch(x + (s + NSLOT) * cells, pre);
@@ -658,7 +655,6 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
         }
         lds_barrier();
         if (active) {
-            float *hs = halo_out + ((long)s * nblk + blk) * TL::NH;
 #pragma unroll
             for (int k = 0; k < NHPT; ++k) {
                 const int hh = pl.lane + k * TL::TPS;
@@ -673,17 +669,21 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
                         acc = fmaf(ent[q].x, d, acc);
                         hw[k][q] = fmaf(xh[k], d, hw[k][q]);
                     }
-                    hs[hh] = acc;
+                    h_done[k] = acc;
                 }
             }
-            if (dx_accumulate) add_cells<CPT>(dx + s * cells + pl.gc, g);
-            else store_cells<CPT>(dx + s * cells + pl.gc, g);
         }
+        done_s = active ? s : -1;
 #pragma unroll
-        for (int c = 0; c < CPT; ++c) g[c] = gnext[c];
+        for (int c = 0; c < CPT; ++c) {
+            g_done[c] = g[c];
+            g[c] = gnext[c];
+        }
         // No barrier here: the next commit writes only the x windows, whose last readers are
         // before the barrier above; delta copy 1 is next written after at least one more barrier.
     }
+
+    flush_done();
 
     // ---- parameter gradients: reduce across slots through LDS, then commit ----
     if (NSLOT > 1) {
@@ -928,7 +928,7 @@ template <int BS, int CPT, int NSLOT, int ACT> int launch_bwd(const StepArgs &a,
 constexpr int kFwdCpt8 = 4, kFwdSlots8 = 1;   // bs=8 forward: 128 threads, 4 cells each
 constexpr int kBwdCpt8 = 2, kBwdSlots8 = 1;   // bs=8 backward: 256 threads, 2 cells each
 constexpr int kFwdCpt4 = 2, kFwdSlots4 = 4;   // bs=4: 32-thread slots, 4 per workgroup
-constexpr int kBwdCpt4 = 2, kBwdSlots4 = 4;
+constexpr int kBwdCpt4 = 1, kBwdSlots4 = 2;   // bs=4 backward: one wave per slot, one cell per thread
 
 template <bool BWD, int ACT> int dispatch_bs(const StepArgs &a, hipStream_t st) {
     if (a.block_size == 8) {
