@@ -1,0 +1,57 @@
+"""The committed C1 fixture (tests/golden/c1_network.npz, written by make_c1_fixture.py from the
+CPU oracle) against the oracle on the CPU and against the HIP path on the GPU."""
+
+import dataclasses
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import assert_close
+
+FIXTURE = os.path.join(os.path.dirname(__file__), "golden", "c1_network.npz")
+NAMES = ("y", "dweight", "dbias", "dscale", "dgamma", "dbeta", "dx0")
+
+
+def c1():
+    from gridnet_amd.configs import WORKLOADS, make_inputs
+
+    wl = dataclasses.replace(WORKLOADS["C1"], backward=True)
+    return wl, make_inputs(wl, seed=0)
+
+
+def test_fixture_inputs_are_the_seeded_ones():
+    _, t = c1()
+    gold = np.load(FIXTURE)
+    assert abs(float(gold["x0_checksum"]) - t["x0"].double().sum().item()) < 1e-9
+
+
+def test_oracle_reproduces_fixture_in_fp32():
+    """ref-style (the reference's op sequence) in fp32 lands on the fp64 fixture within the bar."""
+    from oracle.network import network_forward_backward
+    from oracle.ref_style import gridnet_step_ref
+
+    wl, t = c1()
+    gold = np.load(FIXTURE)
+    out = network_forward_backward(
+        [t[k] for k in ("weight", "bias", "scale", "gamma", "beta")], t["x0"], t["grad_out"],
+        inner_iterations=wl.inner, outer_iterations=wl.outer, block_size=wl.block_size,
+        activation=wl.activation, normalize=wl.normalize, step_fn=gridnet_step_ref)
+    for name, got in zip(NAMES, out):
+        assert_close(got, torch.from_numpy(gold[name]), what=name)
+
+
+@pytest.mark.gpu
+def test_hip_path_reproduces_fixture():
+    from gridnet_amd.runner import BodyRunner
+
+    wl, t = c1()
+    gold = np.load(FIXTURE)
+    d = {k: v.to("cuda:0") for k, v in t.items()}
+    run = BodyRunner(d["weight"], d["bias"], d["scale"], d["gamma"], d["beta"], wl.batch, wl.inner,
+                     wl.outer, wl.block_size, wl.activation, wl.normalize)
+    y = run.forward(d["x0"]).clone()
+    grads = run.backward(d["grad_out"])
+    for name, got in zip(NAMES, (y, *grads)):
+        assert_close(got, torch.from_numpy(gold[name]), what=name)

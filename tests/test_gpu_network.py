@@ -1,0 +1,186 @@
+"""GPU parity of the whole path (outer x (step, LayerNorm), forward and backward) on the
+benchmark workloads, plus size-independent properties at the full training shape."""
+
+import dataclasses
+
+import pytest
+import torch
+
+from oracle.network import network_forward_backward, network_forward
+
+from helpers import assert_close
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+PARAMS = ("weight", "bias", "scale", "gamma", "beta")
+
+
+def runner_for(wl, t, backward=True):
+    from gridnet_amd.runner import BodyRunner
+
+    d = {k: v.to(DEV) for k, v in t.items()}
+    run = BodyRunner(d["weight"], d["bias"], d["scale"], d["gamma"], d["beta"], t["x0"].shape[0],
+                     wl.inner, wl.outer, wl.block_size, wl.activation, wl.normalize,
+                     backward=backward)
+    return run, d
+
+
+def check_against_oracle(wl, t, backward):
+    print(f"workload {wl.name} batch={t['x0'].shape[0]} grid={t['x0'].shape[1]}", flush=True)
+    run, d = runner_for(wl, t, backward)
+    y = run.forward(d["x0"]).clone()
+    kw = dict(inner_iterations=wl.inner, outer_iterations=wl.outer, block_size=wl.block_size,
+              activation=wl.activation, normalize=wl.normalize)
+    if not backward:
+        want = network_forward(*[t[k].double() for k in PARAMS], t["x0"].double(), wl.inner,
+                               wl.outer, wl.block_size, wl.activation, wl.normalize)
+        assert_close(y, want, what="y")
+        return
+    grads = [g.clone() for g in run.backward(d["grad_out"])]
+    want = network_forward_backward([t[k].double() for k in PARAMS], t["x0"].double(),
+                                    t["grad_out"].double(), **kw)
+    names = ("y", "dweight", "dbias", "dscale", "dgamma", "dbeta", "dx0")
+    for name, got, exp in zip(names, (y, *grads), want):
+        assert_close(got, exp, what=name)
+
+
+def test_c1_exact_config_forward_and_backward():
+    from gridnet_amd.configs import WORKLOADS, make_inputs
+
+    wl = dataclasses.replace(WORKLOADS["C1"], backward=True)
+    check_against_oracle(wl, make_inputs(wl), True)
+
+
+@pytest.mark.parametrize("name,grid,batch,outer", [("C2", 32, 4, 3), ("C3", 32, 3, 3),
+                                                   ("C4", 32, 2, 2), ("C5", 16, 5, 2)])
+def test_workload_shapes_reduced(name, grid, batch, outer):
+    """The benchmark workloads with their own block size, inner depth, bias and activation, on a
+    grid/batch/outer count the CPU oracle finishes in seconds."""
+    from gridnet_amd.configs import WORKLOADS, make_inputs
+
+    wl = dataclasses.replace(WORKLOADS[name], grid=grid, batch=batch, outer=outer)
+    if wl.inner >= 8:  # keep 8 residual updates contractive (fp32 rounding otherwise grows)
+        t = make_inputs(wl)
+        t["weight"] = t["weight"] * 0.5
+        t["scale"] = t["scale"] * 0.5
+    else:
+        t = make_inputs(wl)
+    check_against_oracle(wl, t, wl.backward)
+
+
+def test_c3_full_grid_one_outer_step():
+    """The graded shape at its full 64^3 grid and 8^3 blocks (512 blocks: one workgroup owns
+    the whole batch of a block), batch trimmed so that the fp64 oracle stays in seconds."""
+    from gridnet_amd.configs import WORKLOADS, make_inputs
+
+    wl = dataclasses.replace(WORKLOADS["C3"], batch=2, outer=1)
+    check_against_oracle(wl, make_inputs(wl), True)
+
+
+def test_c3_full_size_properties():
+    """Full C3 (batch 32, 12 outer steps): bitwise reproducibility of every output, finiteness,
+    LayerNorm invariants of the result, and batch independence of y and dx."""
+    from gridnet_amd.configs import WORKLOADS, make_inputs
+
+    wl = WORKLOADS["C3"]
+    t = make_inputs(wl)
+    run, d = runner_for(wl, t)
+    y1 = run.forward(d["x0"]).clone()
+    g1 = [g.clone() for g in run.backward(d["grad_out"])]
+    y2 = run.forward(d["x0"]).clone()
+    g2 = [g.clone() for g in run.backward(d["grad_out"])]
+    assert torch.equal(y1, y2)
+    for a, b in zip(g1, g2):
+        assert torch.equal(a, b), "backward is not bitwise reproducible"
+        assert torch.isfinite(a).all()
+    flat = y1.flatten(1)
+    assert flat.mean(1).abs().max().item() < 1e-4          # gamma = 1, beta = 0
+    assert (flat.var(1, unbiased=False) - 1).abs().max().item() < 1e-3
+    # samples do not interact: the first 4 samples alone give the same y and dx for them
+    small = dataclasses.replace(wl, batch=4)
+    ts = {k: (v[:4] if k in ("x0", "grad_out") else v) for k, v in t.items()}
+    run_s, ds = runner_for(small, ts)
+    ys = run_s.forward(ds["x0"]).clone()
+    gs = run_s.backward(ds["grad_out"])
+    assert torch.equal(ys, y1[:4])
+    assert_close(gs[5], g1[5][:4], what="dx0 of a sub-batch")
+    # parameter gradients are sums over the batch: zero upstream gradient on all but 4 samples
+    masked = d["grad_out"].clone()
+    masked[4:] = 0
+    run.forward(d["x0"])
+    gm = run.backward(masked)
+    assert_close(gm[0], gs[0], rtol=1e-4, atol=2e-5, what="dweight restricted to a sub-batch")
+
+
+def test_zero_weights_closed_form_full_size():
+    """w = 0, full C3 step: y = x + T r act(b), whatever the blocking (closed form restated from
+    gridnet/backend_torch_test.py:28-60)."""
+    import gridnet_amd
+    from gridnet_amd.configs import WORKLOADS, make_inputs
+
+    wl = WORKLOADS["C3"]
+    t = make_inputs(wl)
+    x = t["x0"].to(DEV)
+    b, r = t["bias"].to(DEV), torch.full_like(t["bias"], 0.31).to(DEV)
+    y = gridnet_amd.gridnet_step(torch.zeros_like(t["weight"]).to(DEV), b, r, x, wl.inner,
+                                 wl.block_size, 1e-5, False, "silu")
+    want = x + wl.inner * 0.31 * torch.nn.functional.silu(b)
+    assert torch.allclose(y, want, rtol=1e-5, atol=1e-5)
+
+
+def test_graph_replay_matches_eager():
+    """The C-ABI calls only enqueue kernels (no allocation, no synchronisation, fill kernels
+    instead of memsets), so a captured step replays to the eager result every time."""
+    from gridnet_amd.configs import WORKLOADS, make_inputs
+
+    # 64^3 grid: every block's whole batch belongs to one workgroup, so results are bitwise
+    # reproducible (smaller grids split the batch and sum parameter gradients with atomics)
+    wl = dataclasses.replace(WORKLOADS["C3"], batch=4, outer=2)
+    t = make_inputs(wl)
+    run, d = runner_for(wl, t)
+    y_ref = run.forward(d["x0"]).clone()
+    g_ref = [g.clone() for g in run.backward(d["grad_out"])]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        run.forward(d["x0"])
+        run.backward(d["grad_out"])
+        side.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            y_buf = run.forward(d["x0"])
+            g_buf = run.backward(d["grad_out"])
+    for _ in range(3):
+        for g in g_buf:
+            g.fill_(7.0)            # eager work between replays
+        y_buf.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y_buf, y_ref)
+        for a, b in zip(g_buf, g_ref):
+            assert torch.equal(a, b)
+
+
+def test_autograd_body_matches_runner():
+    """GridnetBody (autograd ops, torch-managed memory) and BodyRunner (preallocated) agree."""
+    from gridnet_amd import GridnetBody
+    from gridnet_amd.configs import WORKLOADS, make_inputs
+
+    wl = dataclasses.replace(WORKLOADS["C3"], grid=16, batch=3, outer=2)
+    t = make_inputs(wl)
+    run, d = runner_for(wl, t)
+    y = run.forward(d["x0"]).clone()
+    grads = [g.clone() for g in run.backward(d["grad_out"])]
+    body = GridnetBody((16, 16, 16), wl.inner, wl.outer, wl.block_size, DEV, wl.activation)
+    with torch.no_grad():
+        body.network.weight.copy_(d["weight"])
+        body.network.bias.copy_(d["bias"])
+        body.network.residual_scale.copy_(d["scale"])
+    x = d["x0"].clone().requires_grad_(True)
+    out = body(x)
+    out.backward(d["grad_out"])
+    assert_close(out, y, what="y")
+    assert_close(body.network.weight.grad, grads[0], what="dweight")
+    assert_close(body.norm.weight.grad, grads[3], what="dgamma")
+    assert_close(x.grad, grads[5], what="dx0")
