@@ -13,10 +13,11 @@ import torch
 import torch.nn as nn
 
 try:
-    from .backend_cuda import GridnetCudaOp
+    from .backend_cuda import GatedGridnetCudaOp, GridnetCudaOp
+    from .layernorm import GridLayerNorm, grid_layer_norm
     _IMPORT_ERROR = None
-except ImportError as exc:  # library not built
-    GridnetCudaOp = None
+except ImportError as exc:  # library not built yet (``python -m gridnet_amd.build``) or stale
+    GridnetCudaOp = GatedGridnetCudaOp = GridLayerNorm = grid_layer_norm = None
     _IMPORT_ERROR = exc
 
 SUPPORTED_BLOCK_SIZES = (4, 8)
@@ -41,6 +42,42 @@ def gridnet_step(weight, bias, residual_scale, init_activations, inner_iteration
             f"gridnet block_size {block_size} not supported by the HIP kernels (4 or 8)")
     return GridnetCudaOp.apply(weight, bias, residual_scale, init_activations, inner_iterations,
                                block_size, eps, normalize, activation)
+
+
+def gated_gridnet_step(weight, bias, init_activations, inner_iterations: int, block_size: int,
+                       activation: str = "tanh"):
+    """Gated outer step; signature of gridnet/__init__.py:197-204.  HIP tensors only."""
+    if GatedGridnetCudaOp is None:
+        raise RuntimeError(f"gridnet HIP library is not available: {_IMPORT_ERROR}")
+    if weight.device.type != "cuda":
+        raise NotImplementedError(
+            f"gridnet_amd runs on HIP devices only, got tensors on {weight.device}")
+    if block_size not in SUPPORTED_BLOCK_SIZES:
+        raise NotImplementedError(
+            f"gridnet block_size {block_size} not supported by the HIP kernels (4 or 8)")
+    return GatedGridnetCudaOp.apply(weight, bias, init_activations, inner_iterations, block_size,
+                                    activation)
+
+
+class GatedGridnet(nn.Module):
+    """Parameters and defaults of gridnet/__init__.py:67-99 (same state-dict keys)."""
+
+    def __init__(self, shape: Tuple[int, int, int], inner_iterations: int, block_size: int,
+                 device, dtype=torch.float32, init_scale: float = 1.0, activation: str = "tanh"):
+        super().__init__()
+        self.shape = tuple(shape)
+        self.inner_iterations = inner_iterations
+        self.block_size = block_size
+        self.activation = activation
+        self.weight = nn.Parameter(
+            torch.randn(27, 2, *shape, device=device, dtype=dtype) * (init_scale / math.sqrt(27)))
+        self.bias = nn.Parameter(torch.zeros(2, *shape, device=device, dtype=dtype))
+        self.device = device
+        self.dtype = dtype
+
+    def forward(self, x):
+        return gated_gridnet_step(self.weight, self.bias, x, self.inner_iterations,
+                                  self.block_size, self.activation)
 
 
 class Gridnet(nn.Module):
@@ -70,8 +107,7 @@ class Gridnet(nn.Module):
                             self.activation)
 
 
-from .layernorm import GridLayerNorm, grid_layer_norm  # noqa: E402
 from .network import GridnetBody  # noqa: E402
 
-__all__ = ["gridnet_step", "Gridnet", "GridnetCudaOp", "GridLayerNorm", "grid_layer_norm",
-           "GridnetBody"]
+__all__ = ["gridnet_step", "gated_gridnet_step", "Gridnet", "GatedGridnet", "GridnetCudaOp",
+           "GatedGridnetCudaOp", "GridLayerNorm", "grid_layer_norm", "GridnetBody"]

@@ -55,3 +55,40 @@ class GridnetCudaOp(torch.autograd.Function):
                               bias_grad, residual_scale_grad, x_grad, ctx.inner_iters,
                               ctx.block_size, ctx.eps, ctx.normalize, ctx.activation)
         return (weight_grad, bias_grad, residual_scale_grad, x_grad, None, None, None, None, None)
+
+
+class GatedGridnetCudaOp(torch.autograd.Function):
+    """Mirror of gridnet/backend_cuda.py:111-190: six positional ``apply`` arguments."""
+
+    @staticmethod
+    def forward(ctx, weight, bias, init_activations, inner_iters: int, block_size: int,
+                activation: str):
+        x = init_activations
+        batch_size, m, n, k = x.shape
+        assert m % block_size == 0 and n % block_size == 0 and k % block_size == 0, (
+            f"{block_size=} incompatible with {x.shape=}")
+        assert weight.shape == (27, 2, m, n, k), f"{weight.shape=} invalid for {x.shape=}"
+        assert bias.shape == weight.shape[1:], f"{bias.shape=} invalid for {weight.shape=}"
+        assert weight.dtype == bias.dtype, f"mismatching dtypes: {weight.dtype=} {bias.dtype=}"
+        assert weight.dtype == x.dtype, f"mismatching dtypes: {weight.dtype=} {x.dtype=}"
+        assert weight.device == bias.device, f"mismatching devices: {weight.device=} {bias.device=}"
+        assert weight.device == x.device, f"mismatching devices: {weight.device=} {x.device=}"
+        if not batch_size:
+            return x.clone()
+        ctx.save_for_backward(weight, bias, x)
+        ctx.inner_iters = inner_iters
+        ctx.block_size = block_size
+        ctx.activation = activation
+        outputs = torch.empty_like(x)
+        gridnet_cuda.forward_gated(weight, bias, x, outputs, inner_iters, block_size, activation)
+        return outputs
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        weight, bias, x = ctx.saved_tensors
+        weight_grad = torch.zeros_like(weight)
+        bias_grad = torch.zeros_like(bias)
+        x_grad = torch.zeros_like(x)
+        gridnet_cuda.backward_gated(weight, bias, x, grad_output, weight_grad, bias_grad, x_grad,
+                                    ctx.inner_iters, ctx.block_size, ctx.activation)
+        return (weight_grad, bias_grad, x_grad, None, None, None)

@@ -30,7 +30,7 @@ int check_launch(const char *what) {
 
 namespace {
 
-int check_step(const StepArgs &a, bool backward) {
+int check_step(const StepArgs &a, bool backward, bool gated = false) {
     if (a.dtype != GRIDNET_F32 && a.dtype != GRIDNET_F64)
         return fail(GRIDNET_ERR_ARGUMENT, "unsupported dtype id %d", a.dtype);
     if (a.B < 0 || a.M <= 0 || a.N <= 0 || a.K <= 0)
@@ -49,10 +49,10 @@ int check_step(const StepArgs &a, bool backward) {
     if ((long)a.M * a.N * a.K * 27 >= (1L << 31))
         return fail(GRIDNET_ERR_ARGUMENT, "grid too large: 27*M*N*K must be below 2^31");
     if (a.B == 0) return GRIDNET_OK;
-    if (!a.weight || !a.bias || !a.scale || !a.x)
+    if (!a.weight || !a.bias || (!a.scale && !gated) || !a.x)
         return fail(GRIDNET_ERR_ARGUMENT, "null input pointer");
     if (!backward && !a.y) return fail(GRIDNET_ERR_ARGUMENT, "null output pointer");
-    if (backward && (!a.dy || !a.dweight || !a.dbias || !a.dscale || !a.dx))
+    if (backward && (!a.dy || !a.dweight || !a.dbias || (!a.dscale && !gated) || !a.dx))
         return fail(GRIDNET_ERR_ARGUMENT, "null gradient pointer");
     return GRIDNET_OK;
 }
@@ -125,6 +125,34 @@ int gridnet_hip_backward(int dtype, const void *weight, const void *bias, const 
         return step_backward_fast(a, st);
     }
     return step_backward_generic(a, st);
+}
+
+int gridnet_hip_forward_gated(int dtype, const void *weight, const void *bias, const void *x, void *y,
+                              int B, int M, int N, int K, int inner, int block_size, int activation,
+                              void *stream) {
+    StepArgs a{};
+    a.dtype = dtype; a.weight = weight; a.bias = bias; a.x = x; a.y = y;
+    a.B = B; a.M = M; a.N = N; a.K = K; a.inner = inner; a.block_size = block_size;
+    a.activation = activation;
+    if (int rc = check_step(a, false, true)) return rc;
+    if (B == 0) return GRIDNET_OK;
+    return gated_forward(a, (hipStream_t)stream);
+}
+
+int gridnet_hip_backward_gated(int dtype, const void *weight, const void *bias, const void *x,
+                               const void *dy, void *dweight, void *dbias, void *dx, int B, int M,
+                               int N, int K, int inner, int block_size, int activation, int flags,
+                               void *stream) {
+    StepArgs a{};
+    a.dtype = dtype; a.weight = weight; a.bias = bias; a.x = x; a.dy = dy;
+    a.dweight = dweight; a.dbias = dbias; a.dx = dx;
+    a.B = B; a.M = M; a.N = N; a.K = K; a.inner = inner; a.block_size = block_size;
+    a.activation = activation; a.flags = flags;
+    if (int rc = check_step(a, true, true)) return rc;
+    if ((long)M * N * K * 54 >= (1L << 31))
+        return fail(GRIDNET_ERR_ARGUMENT, "grid too large: 54*M*N*K must be below 2^31");
+    if (B == 0) return GRIDNET_OK;
+    return gated_backward(a, (hipStream_t)stream);
 }
 
 size_t gridnet_hip_layernorm_workspace_bytes(int dtype, int B, long n) {

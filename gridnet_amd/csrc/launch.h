@@ -49,6 +49,10 @@ size_t step_fast_backward_workspace(const StepArgs &a);
 int step_forward_fast(const StepArgs &a, hipStream_t st);
 int step_backward_fast(const StepArgs &a, hipStream_t st);
 
+// gated_generic.hip (weight [27,2,M,N,K], bias [2,M,N,K]; scale, eps, normalize unused)
+int gated_forward(const StepArgs &a, hipStream_t st);
+int gated_backward(const StepArgs &a, hipStream_t st);
+
 // layernorm.hip
 size_t layernorm_workspace(int dtype, int B, long n);
 int layernorm_forward(const LayerNormArgs &a, hipStream_t st);

@@ -27,6 +27,8 @@ EXPORTS = (
     "gridnet_hip_forward",
     "gridnet_hip_backward_workspace_bytes",
     "gridnet_hip_backward",
+    "gridnet_hip_forward_gated",
+    "gridnet_hip_backward_gated",
     "gridnet_hip_layernorm_workspace_bytes",
     "gridnet_hip_layernorm_forward",
     "gridnet_hip_layernorm_backward",
@@ -57,6 +59,10 @@ def _load():
     lib.gridnet_hip_backward.restype = i
     lib.gridnet_hip_backward.argtypes = [i, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, d, i, i, i,
                                          p, z, p]
+    lib.gridnet_hip_forward_gated.restype = i
+    lib.gridnet_hip_forward_gated.argtypes = [i, p, p, p, p, i, i, i, i, i, i, i, p]
+    lib.gridnet_hip_backward_gated.restype = i
+    lib.gridnet_hip_backward_gated.argtypes = [i, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, p]
     lib.gridnet_hip_layernorm_workspace_bytes.restype = z
     lib.gridnet_hip_layernorm_workspace_bytes.argtypes = [i, i, l]
     lib.gridnet_hip_layernorm_forward.restype = i
@@ -66,7 +72,10 @@ def _load():
     return lib
 
 
-lib = _load()
+try:
+    lib = _load()
+except AttributeError as exc:  # an older build of the library without some entry point
+    raise ImportError(f"{LIB_PATH} is stale ({exc}): rebuild with `python -m gridnet_amd.build`") from exc
 
 
 def last_error() -> str:

@@ -60,11 +60,32 @@ def backward(weight, bias, scale, initActivations, outGrads, weightGradOut, bias
 
 def forward_gated(weight, bias, initActivations, outActivations, innerIterations, blockSize,
                   activation):
-    """Gated variant (src/gridnet_cuda.cpp:133-158): not part of this library yet."""
-    raise NotImplementedError("gridnet_cuda.forward_gated is not provided by libgridnet_hip")
+    """Gated outer step; replaces gated_gridnet_forward, src/gridnet_cuda.cpp:133-158."""
+    for t, name in ((weight, "weight"), (bias, "bias"), (initActivations, "initActivations"),
+                    (outActivations, "outActivations")):
+        _n.check_input(t, name)
+    act = _n.activation_id(activation)
+    B, M, N, K = initActivations.shape
+    with torch.cuda.device(weight.device):
+        _n.check(_n.lib.gridnet_hip_forward_gated(
+            _n.dtype_id(weight), weight.data_ptr(), bias.data_ptr(), initActivations.data_ptr(),
+            outActivations.data_ptr(), B, M, N, K, int(innerIterations), int(blockSize), act,
+            _n.current_stream(weight)))
 
 
 def backward_gated(weight, bias, initActivations, outGrads, weightGradOut, biasGradOut,
                    activationsGradOut, innerIterations, blockSize, activation):
-    """Gated variant (src/gridnet_cuda.cpp:160-186): not part of this library yet."""
-    raise NotImplementedError("gridnet_cuda.backward_gated is not provided by libgridnet_hip")
+    """Backward of the gated step; replaces gated_gridnet_backward, src/gridnet_cuda.cpp:160-186.
+    Gradient outputs are accumulated into, as in the reference."""
+    for t, name in ((weight, "weight"), (bias, "bias"), (initActivations, "initActivations"),
+                    (outGrads, "outGrads"), (weightGradOut, "weightGradOut"),
+                    (biasGradOut, "biasGradOut"), (activationsGradOut, "activationsGradOut")):
+        _n.check_input(t, name)
+    act = _n.activation_id(activation)
+    B, M, N, K = initActivations.shape
+    with torch.cuda.device(weight.device):
+        _n.check(_n.lib.gridnet_hip_backward_gated(
+            _n.dtype_id(weight), weight.data_ptr(), bias.data_ptr(), initActivations.data_ptr(),
+            outGrads.data_ptr(), weightGradOut.data_ptr(), biasGradOut.data_ptr(),
+            activationsGradOut.data_ptr(), B, M, N, K, int(innerIterations), int(blockSize), act, 0,
+            _n.current_stream(weight)))

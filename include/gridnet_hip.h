@@ -97,6 +97,23 @@ int gridnet_hip_backward(int dtype, const void *weight, const void *bias, const 
                          void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * Gated variant: x' = gate*x + (1-gate)*act(pre), weight [27,2,M,N,K] (channel 0: pre,
+ * channel 1: gate), bias [2,M,N,K]; no scale, eps or normalisation.  Replace
+ * gated_gridnet_cuda_forward / gated_gridnet_cuda_backward, src/gridnet_cuda_kernels.cu:853-930
+ * (bound as `forward_gated` / `backward_gated`, src/gridnet_cuda.cpp:133-186,192-193).
+ * Backward: inner <= 32; dweight [27,2,M,N,K], dbias [2,M,N,K] summed over the batch; flags as
+ * for gridnet_hip_backward.  No workspace.
+ */
+int gridnet_hip_forward_gated(int dtype, const void *weight, const void *bias, const void *x,
+                              void *y, int B, int M, int N, int K, int inner, int block_size,
+                              int activation, void *stream);
+
+int gridnet_hip_backward_gated(int dtype, const void *weight, const void *bias, const void *x,
+                               const void *dy, void *dweight, void *dbias, void *dx, int B, int M,
+                               int N, int K, int inner, int block_size, int activation, int flags,
+                               void *stream);
+
+/*
  * Per-sample LayerNorm over all n = M*N*K cells with elementwise affine, the op the callers
  * place after every outer step (torch.nn.LayerNorm((M,N,K)): gridnet/scripts/train_mnist.py:54,64,
  * gridnet/scripts/train_imagenet.py:67,86).  y = (x-mean)*rstd*gamma + beta, biased variance,
