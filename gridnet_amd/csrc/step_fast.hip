@@ -554,27 +554,53 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
         fx.fetch(x + (s0 + pl.slot) * cells, pre);
         load_cells<CPT>(dy + (s0 + pl.slot) * cells + pl.gc, g);
     }
-    // The gradients of an element leave one element late, after the next window has been
-    // committed: the wait for the prefetched window would otherwise also wait for stores that
-    // were issued an instant earlier (loads and stores share one in-order counter).
-    float g_done[CPT], h_done[NHPT];
+    // Per element: commit its window, barrier, [halo pass and stores of the PREVIOUS element],
+    // recompute, reverse sweep, write D = sum_i delta_i into delta copy 1, commit the next
+    // window.  Deferring the halo pass past the next barrier saves a barrier per element, lets
+    // its dependent LDS look-ups overlap the first stencil loads of the next element, and keeps
+    // the stores away from the wait on the prefetched window (loads and stores share one
+    // in-order counter).
+    float g_done[CPT], xh[NHPT], xh_done[NHPT];
     int done_s = -1;
-    auto flush_done = [&]() {
+    auto finish_done = [&]() {  // call only after a barrier that follows the D write
         if (done_s < 0) return;
         float *hs = halo_out + ((long)done_s * nblk + blk) * TL::NH;
 #pragma unroll
-        for (int k = 0; k < NHPT; ++k)
-            if (pl.lane + k * TL::TPS < TL::NH) hs[pl.lane + k * TL::TPS] = h_done[k];
+        for (int k = 0; k < NHPT; ++k) {
+            const int hh = pl.lane + k * TL::TPS;
+            if (hh < TL::NH) {
+                float2 ent[TL::NPAIR];
+#pragma unroll
+                for (int q = 0; q < TL::NPAIR; ++q) ent[q] = tab[hh * TL::NPAIR + q];
+                float acc = 0.f;
+#pragma unroll
+                for (int q = 0; q < TL::NPAIR; ++q) {
+                    const float d = dwin[TL::WIN + __float_as_int(ent[q].y)];
+                    acc = fmaf(ent[q].x, d, acc);
+                    hw[k][q] = fmaf(xh_done[k], d, hw[k][q]);
+                }
+                hs[hh] = acc;
+            }
+        }
         if (dx_accumulate) add_cells<CPT>(dx + done_s * cells + pl.gc, g_done);
         else store_cells<CPT>(dx + done_s * cells + pl.gc, g_done);
         done_s = -1;
     };
+    if (s0 + pl.slot < s1) fx.commit(win, pre);
+#ifdef EXP_TIMING
+    long t_acc[5] = {0, 0, 0, 0, 0};
+    long t_prev = clock64();
+#define TICK(i) { long t_now = clock64(); t_acc[i] += t_now - t_prev; t_prev = t_now; }
+#else
+#define TICK(i)
+#endif
     for (int sb = s0; sb < s1; sb += NSLOT) {
         const int s = sb + pl.slot;
         const bool active = s < s1;  // a slot past the end idles through the barriers
-        if (active) fx.commit(win, pre);
-        lds_barrier();
-        flush_done();
+        lds_barrier();               // this element's window and the previous element's D
+        TICK(0)
+        finish_done();
+        TICK(1)
         float gnext[CPT];
         if (s + NSLOT < s1) {
             fx.fetch(x + (s + NSLOT) * cells, pre);
@@ -584,6 +610,9 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
         if (active) {
 #pragma unroll
             for (int c = 0; c < CPT; ++c) cur[c] = win[pl.own + c];
+            // x on the halo (identical in both window copies, frozen for the whole element)
+#pragma unroll
+            for (int k = 0; k < NHPT; ++k) xh[k] = win[hoff[k]];
         }
 
         // ---- forward recompute, remembering x_i and u_i of the owned cells ----
@@ -605,6 +634,7 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
             if (it + 1 < inner) lds_barrier();
         }
 
+        TICK(2)
         // ---- reverse sweep: delta window copy (it & 1) holds delta_it ----
         float dsum[CPT], xi[CPT];
 #pragma unroll
@@ -641,37 +671,15 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
             }
         }
 
-        // ---- cells of the neighbouring blocks: one gather pass over D = sum_i delta_i.
-        // Delta copy 1 is free: the last iteration (it = 0) used copy 0, and the readers of
-        // copy 1 (it = 1) are past the barrier of it = 0.
-        float xh[NHPT];
+        TICK(3)
+        // ---- cells of the neighbouring blocks need only D = sum_i delta_i (the halo is frozen);
+        // D goes to delta copy 1: the last iteration (it = 0) used copy 0 and the readers of
+        // copy 1 (it = 1) are past the barrier of it = 0.  The pass itself runs after the next
+        // barrier (finish_done).
+        if (inner == 0) lds_barrier();  // no barrier since the top: others may still read LDS
         if (active) {
 #pragma unroll
             for (int c = 0; c < CPT; ++c) dwin[TL::WIN + pl.own + c] = dsum[c];
-            // x on the halo (identical in both window copies), read before the barrier so that
-            // the next element's window may be committed right after it
-#pragma unroll
-            for (int k = 0; k < NHPT; ++k) xh[k] = win[hoff[k]];
-        }
-        lds_barrier();
-        if (active) {
-#pragma unroll
-            for (int k = 0; k < NHPT; ++k) {
-                const int hh = pl.lane + k * TL::TPS;
-                if (hh < TL::NH) {
-                    float2 ent[TL::NPAIR];
-#pragma unroll
-                    for (int q = 0; q < TL::NPAIR; ++q) ent[q] = tab[hh * TL::NPAIR + q];
-                    float acc = 0.f;
-#pragma unroll
-                    for (int q = 0; q < TL::NPAIR; ++q) {
-                        const float d = dwin[TL::WIN + __float_as_int(ent[q].y)];
-                        acc = fmaf(ent[q].x, d, acc);
-                        hw[k][q] = fmaf(xh[k], d, hw[k][q]);
-                    }
-                    h_done[k] = acc;
-                }
-            }
         }
         done_s = active ? s : -1;
 #pragma unroll
@@ -679,11 +687,18 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
             g_done[c] = g[c];
             g[c] = gnext[c];
         }
-        // No barrier here: the next commit writes only the x windows, whose last readers are
-        // before the barrier above; delta copy 1 is next written after at least one more barrier.
+#pragma unroll
+        for (int k = 0; k < NHPT; ++k) xh_done[k] = xh[k];
+        // the x windows are free (the reverse sweep does not read them): commit the next one
+        if (s + NSLOT < s1) fx.commit(win, pre);
+        TICK(4)
     }
-
-    flush_done();
+    lds_barrier();
+    finish_done();
+#ifdef EXP_TIMING
+    if (threadIdx.x == 0)
+        for (int i = 0; i < 5; ++i) halo_out[blk * 8 + i] = (float)t_acc[i];
+#endif
 
     // ---- parameter gradients: reduce across slots through LDS, then commit ----
     if (NSLOT > 1) {
