@@ -51,47 +51,8 @@ template <int BS, int CPT> struct Tile {
     static constexpr int PS = S * RS;             // LDS plane stride
     static constexpr int WIN = S * PS;            // floats per window copy
     static constexpr int NWIN = S * S * S;        // window entries
-    static constexpr int NLOAD = (NWIN + TPS - 1) / TPS;  // window entries fetched per thread
-    static constexpr int MID = 4 * S - 4;         // halo entries of a middle plane
-    static constexpr int NH = 2 * S * S + BS * MID;  // halo entries of a window
-    static constexpr int NPAIR = 9;               // (source, weight) pairs per halo entry
     static_assert(BS % CPT == 0, "cells per thread must divide the block side");
 };
-
-// Compact numbering of the halo: the two full planes i=0 and i=S-1, then for each middle plane
-// the rows j=0 and j=S-1 and the two end cells of every other row.
-template <typename TL>
-__host__ __device__ __forceinline__ void halo_coords(int h, int &wi, int &wj, int &wk) {
-    constexpr int S = TL::S, P = S * S;
-    if (h < 2 * P) {
-        wi = h < P ? 0 : S - 1;
-        const int r = h < P ? h : h - P;
-        wj = r / S;
-        wk = r % S;
-    } else {
-        h -= 2 * P;
-        wi = 1 + h / TL::MID;
-        int r = h % TL::MID;
-        if (r < 2 * S) {
-            wj = r < S ? 0 : S - 1;
-            wk = r < S ? r : r - S;
-        } else {
-            r -= 2 * S;
-            wj = 1 + r / 2;
-            wk = (r & 1) * (S - 1);
-        }
-    }
-}
-
-template <typename TL> __host__ __device__ __forceinline__ int halo_index(int wi, int wj, int wk) {
-    constexpr int S = TL::S, P = S * S;
-    if (wi == 0) return wj * S + wk;
-    if (wi == S - 1) return P + wj * S + wk;
-    const int base = 2 * P + (wi - 1) * TL::MID;
-    if (wj == 0) return base + wk;
-    if (wj == S - 1) return base + S + wk;
-    return base + 2 * S + (wj - 1) * 2 + (wk == S - 1 ? 1 : 0);
-}
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits for every global
 // load in flight, which would stall each inner iteration on the prefetch of the next batch
@@ -197,71 +158,70 @@ template <typename TL, int CPT, int NSLOT> struct Place {
     }
 };
 
-// Fetching a window: one thread per window row (S*S rows of S entries; the first S*S threads
-// of a slot take one row each, or several when the slot is small).  The bs cells of the block
-// that lie in a row are contiguous and 16-byte aligned in the grid, so they come in as float4;
-// the two end entries belong to the neighbouring blocks (or lie outside the grid and read as
-// zero, gridnet/backend_torch.py:63).
+// Fetching a window: one thread per HALF window row (2*S*S half rows of S/2 entries; the first
+// threads of a slot take one each, or several when the slot is small).  A half row is one end
+// entry plus bs/2 cells of the block; the cells are contiguous and 16-byte (bs=8) or 8-byte
+// (bs=4) aligned in the grid and come in as one vector.  End entries belong to the
+// neighbouring blocks, or lie outside the grid and read as zero (gridnet/backend_torch.py:63).
 template <typename TL> struct Fetch {
-    static constexpr int S = TL::S, BS = TL::S - 2;
-    static constexpr int NROW = S * S;
-    static constexpr int RPT = (NROW + TL::TPS - 1) / TL::TPS;  // rows per thread
-    int goff[RPT];   // grid offset (within a sample) of the row's first block cell; off-grid rows
-                     // point at a valid address and are zeroed when committed
-    int loff[RPT];   // LDS offset of the row's first entry, -1: no row for this thread
+    static constexpr int S = TL::S, BS = TL::S - 2, HL = S / 2, HC = BS / 2;
+    static constexpr int NHALF = 2 * S * S;
+    static constexpr int RPT = (NHALF + TL::TPS - 1) / TL::TPS;  // half rows per thread
+    int goff[RPT];   // grid offset (within a sample) of the half row's first block cell; rows
+                     // outside the grid point at a valid address and are zeroed when committed
+    int loff[RPT];   // LDS offset of the half row's first entry, -1: none for this thread
+    int edge[RPT];   // address delta of the end entry relative to goff (0 when it is off-grid)
     bool ok[RPT];    // the row lies inside the grid
-    int lo_d, hi_d;  // address deltas of the two end entries (0 when they are off-grid)
-    bool lo_ok, hi_ok;
+    bool edge_ok[RPT];
+    bool hi[RPT];    // second half: [cells..., end entry] instead of [end entry, cells...]
     __device__ __forceinline__ Fetch(int lane, int p0, int q0, int r0, int M, int N, int K) {
-        lo_ok = r0 > 0;
-        hi_ok = r0 + BS < K;
-        lo_d = lo_ok ? -1 : 0;
-        hi_d = hi_ok ? BS : 0;
 #pragma unroll
         for (int e = 0; e < RPT; ++e) {
-            const int row = lane + e * TL::TPS;
+            const int id = lane + e * TL::TPS;
+            const int half = id & 1, row = id >> 1;
             const int wj = row % S, wi = row / S;
             const int gi = p0 + wi - 1, gj = q0 + wj - 1;
-            const bool have = row < NROW;
+            const bool have = id < NHALF;
+            hi[e] = half != 0;
             ok[e] = have && gi >= 0 && gi < M && gj >= 0 && gj < N;
-            loff[e] = have ? wi * TL::PS + wj * TL::RS : -1;
+            edge_ok[e] = half ? (r0 + BS < K) : (r0 > 0);
+            edge[e] = edge_ok[e] ? (half ? HC : -1) : 0;
+            loff[e] = have ? wi * TL::PS + wj * TL::RS + half * HL : -1;
             // rows outside the grid (and threads without a row) read row (0, 0) of the sample at
-            // the block's own columns: always in bounds, also for the two end entries, because
-            // lo_d / hi_d are non-zero only when columns r0-1 / r0+bs exist
-            goff[e] = ok[e] ? (gi * N + gj) * K + r0 : r0;
+            // the block's own columns: in bounds, also for the end entry, whose delta is
+            // non-zero only when that column exists
+            goff[e] = (ok[e] ? (gi * N + gj) * K : 0) + r0 + half * HC;
         }
     }
     // Unconditional loads (no branches, no register initialisation in front of them).
-    __device__ __forceinline__ void fetch(const float *xs, float (&v)[RPT][S]) const {
+    __device__ __forceinline__ void fetch(const float *xs, float (&v)[RPT][HL]) const {
 #pragma unroll
         for (int e = 0; e < RPT; ++e) {
             const float *p = xs + goff[e];
+            float c[HC];
+            load_cells<HC>(p, c);
+            const float end = p[edge[e]];
+            // lay the values out in window order for either half
 #pragma unroll
-            for (int q = 0; q < BS / 4; ++q) {
-                const float4 t = *reinterpret_cast<const float4 *>(p + 4 * q);
-                v[e][1 + 4 * q] = t.x; v[e][2 + 4 * q] = t.y; v[e][3 + 4 * q] = t.z; v[e][4 + 4 * q] = t.w;
-            }
-            v[e][0] = p[lo_d];
-            v[e][S - 1] = p[hi_d];
+            for (int q = 0; q < HC; ++q) v[e][q] = c[q];
+            v[e][HC] = end;
         }
     }
     // Both window copies receive every entry (the halo must be in both; the block itself is
-    // overwritten by the iterations anyway).  Row starts are 8-byte aligned.
-    __device__ __forceinline__ void commit(float *win, const float (&v)[RPT][S]) const {
+    // overwritten by the iterations anyway).
+    template <int COPIES = 2>
+    __device__ __forceinline__ void commit(float *win, const float (&v)[RPT][HL]) const {
 #pragma unroll
         for (int e = 0; e < RPT; ++e)
             if (loff[e] >= 0) {
-                float r[S];
+                const float end = (ok[e] && edge_ok[e]) ? v[e][HC] : 0.f;
 #pragma unroll
-                for (int q = 0; q < S; ++q) r[q] = ok[e] ? v[e][q] : 0.f;
-                if (!lo_ok) r[0] = 0.f;
-                if (!hi_ok) r[S - 1] = 0.f;
-#pragma unroll
-                for (int copy = 0; copy < 2; ++copy) {
+                for (int copy = 0; copy < COPIES; ++copy) {
                     float *row = win + copy * TL::WIN + loff[e];
+                    // first half: [end, cells...]; second half: [cells..., end]
+                    row[hi[e] ? HC : 0] = end;
 #pragma unroll
-                    for (int q = 0; q < S / 2; ++q)
-                        *reinterpret_cast<float2 *>(row + 2 * q) = make_float2(r[2 * q], r[2 * q + 1]);
+                    for (int q = 0; q < HC; ++q) row[q + (hi[e] ? 0 : 1)] = ok[e] ? v[e][q] : 0.f;
                 }
             }
     }
@@ -343,7 +303,7 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_fwd_fast(
     wait_global_loads();
 
     const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
-    float pre[Fetch<TL>::RPT][TL::S];
+    float pre[Fetch<TL>::RPT][Fetch<TL>::HL];
     if (s0 + pl.slot < s1) fx.fetch(x + (s0 + pl.slot) * cells, pre);
     // The result of an element is stored one element late, after the next window has been
     // committed: the wait for the prefetched window would otherwise also wait for a store that
@@ -386,90 +346,47 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_fwd_fast(
 constexpr int kBwdDepth = 4;  // neighbour rows requested ahead of the arithmetic
 
 // LDS layout of the backward kernel (floats): per slot [x window x2 | delta window x2 |
-// history: inner slabs of TPS*2*CPT], then one table per workgroup [NH*9 weights | NH*9 offsets].
+// history: inner slabs of TPS*2*CPT].
 template <int BS, int CPT> __host__ __device__ constexpr int bwd_slot_floats(int inner) {
     return 4 * Tile<BS, CPT>::WIN + inner * Tile<BS, CPT>::TPS * 2 * CPT;
 }
 template <int BS, int CPT, int NSLOT> size_t bwd_lds_bytes(int inner) {
-    using TL = Tile<BS, CPT>;
-    return ((size_t)NSLOT * bwd_slot_floats<BS, CPT>(inner) + 2 * (size_t)TL::NH * TL::NPAIR) *
-           sizeof(float);
+    return (size_t)NSLOT * bwd_slot_floats<BS, CPT>(inner) * sizeof(float);
 }
 
-// Pair q (0..8) of halo entry h: the block cell `src` (window coordinates) whose tap `t` reads
-// that halo entry.  Every window axis either pins the source (entry on a window face: the
-// adjacent layer of the block) or is free (source at -1, 0, +1 along it); the free axes consume
-// the two base-3 digits of q in order, unused digits must be 1 so each pair appears once.
-template <typename TL, int BS>
-__device__ __forceinline__ bool halo_pair(int h, int q, int &t, int (&src)[3]) {
-    int wc[3];
-    halo_coords<TL>(h, wc[0], wc[1], wc[2]);
-    const int d0 = q / 3, d1 = q % 3;
-    int used = 0;
-    bool valid = true;
+// Commit R x C gradient values to base[index(r, c)] for the entries with ok(r, c).  One code path
+// per mode (the mode is uniform).  In the add-in-place mode the accumulators were STARTED from
+// the old contents (see the kernels' set-up), so that mode stores like the overwrite mode: an
+// old value fetched at the end instead would put a serial trip to memory at the tail of every
+// workgroup, where nothing is left to hide it.
+template <int R, int C, typename Index, typename Ok>
+__device__ __forceinline__ void commit_grads(float *base, const float (&val)[R][C], int mode,
+                                             Index &&index, Ok &&ok) {
+    if (mode != kParamAtomic) {
 #pragma unroll
-    for (int ax = 0; ax < 3; ++ax) {
-        if (wc[ax] == 0) {
-            src[ax] = 1;
-        } else if (wc[ax] == TL::S - 1) {
-            src[ax] = BS;
-        } else {  // a halo entry has at most two free axes
-            src[ax] = wc[ax] + (used == 0 ? d0 : d1) - 1;
-            ++used;
-            valid = valid && src[ax] >= 1 && src[ax] <= BS;
-        }
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+                if (ok(r, c)) base[index(r, c)] = val[r][c];
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+                if (ok(r, c)) unsafeAtomicAdd(base + index(r, c), val[r][c]);
     }
-    if (used < 2) valid = valid && d1 == 1;
-    if (used < 1) valid = valid && d0 == 1;
-    // halo entry = source + off_t  =>  tap digits = entry - source + 1
-    t = (wc[0] - src[0] + 1) * 9 + (wc[1] - src[1] + 1) * 3 + (wc[2] - src[2] + 1);
-    return valid;
-}
-
-// The decode of every (halo entry, pair) is the same for all workgroups and all calls: it is
-// evaluated once per process into a device table, one word per pair:
-// bit 31 = valid, bits 16..20 = tap, bits 0..15 = LDS offset of the source cell in a window.
-__device__ int g_pair_words8[Tile<8, 1>::NH * Tile<8, 1>::NPAIR];
-__device__ int g_pair_words4[Tile<4, 1>::NH * Tile<4, 1>::NPAIR];
-template <int BS> __device__ __forceinline__ int *pair_words() {
-    if constexpr (BS == 8) return g_pair_words8;
-    else return g_pair_words4;
-}
-template <int BS> __global__ void build_pair_words() {
-    using TL = Tile<BS, 1>;
-    const int e = blockIdx.x * blockDim.x + threadIdx.x;
-    if (e >= TL::NH * TL::NPAIR) return;
-    int t, src[3];
-    const bool valid = halo_pair<TL, BS>(e / TL::NPAIR, e % TL::NPAIR, t, src);
-    pair_words<BS>()[e] = valid ? (int)(0x80000000u | (unsigned)(t << 16) |
-                                        (unsigned)(src[0] * TL::PS + src[1] * TL::RS + src[2]))
-                                : 0;
-}
-// Grid index (within a sample) of the source cell of a pair word, for a block at (p0, q0, r0).
-template <typename TL>
-__device__ __forceinline__ int pair_source_cell(int word, int p0, int q0, int r0, int N, int K) {
-    const int off = word & 0xffff;
-    const int s0 = off / TL::PS, s1 = (off % TL::PS) / TL::RS, s2 = off % TL::RS;
-    return ((p0 + s0 - 1) * N + (q0 + s1 - 1)) * K + (r0 + s2 - 1);
-}
-
-__device__ __forceinline__ void commit_grad(float *p, float v, int mode) {
-    if (mode == kParamStore) *p = v;
-    else if (mode == kParamAddExclusive) *p += v;
-    else unsafeAtomicAdd(p, v);
 }
 
 template <int BS, int CPT, int NSLOT, int ACT>
-__global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
+__global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) __attribute__((amdgpu_waves_per_eu(2)))
+void step_bwd_fast(
     const float *__restrict__ weight, const float *__restrict__ bias,
     const float *__restrict__ scale, const float *__restrict__ x, const float *__restrict__ dy,
     float *__restrict__ dweight, float *__restrict__ dbias, float *__restrict__ dscale,
-    float *__restrict__ dx, float *__restrict__ halo_out, int B, int M, int N, int K, int inner,
+    float *__restrict__ dx, float *__restrict__ dsum_out, int B, int M, int N, int K, int inner,
     int nblk, int nchunk, int chunk_len, int param_mode, int dx_accumulate) {
     using TL = Tile<BS, CPT>;
     extern __shared__ __attribute__((aligned(16))) float lds[];
-    constexpr int NT = TL::TPS * NSLOT;
-    constexpr int NHPT = (TL::NH + TL::TPS - 1) / TL::TPS;  // halo entries per thread
     const int slot_floats = bwd_slot_floats<BS, CPT>(inner);
 
     int blk, chunk;
@@ -479,11 +396,18 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
     float *win = lds + pl.slot * slot_floats;
     float *dwin = win + 2 * TL::WIN;
     float *hist = dwin + 2 * TL::WIN + pl.lane * CPT;  // + it*TPS*2*CPT (x_i), + TPS*CPT more (u_i)
-    // per workgroup: (weight, source offset) of every pair, 8 bytes each
-    float2 *tab = reinterpret_cast<float2 *>(lds + NSLOT * slot_floats);
     const long cells = (long)M * N * K;
 
-    // ---- once per workgroup: parameters, mirrored neighbour weights, halo table ----
+    // nw[t][c] belongs to the weight of the neighbour at c + off_t, where that lies in this block
+    auto in_block = [&](int t, int c) {
+        const int ni = pl.i + t / 9 - 1, nj = pl.j + (t / 3) % 3 - 1, nk = pl.kt * CPT + c + t % 3 - 1;
+        return ni >= 0 && ni < BS && nj >= 0 && nj < BS && nk >= 0 && nk < BS;
+    };
+    auto neighbour_weight = [&](int t, int c) {
+        return (26 - t) * cells + pl.gc + c + ((t / 9 - 1) * N + ((t / 3) % 3 - 1)) * K + (t % 3 - 1);
+    };
+
+    // ---- once per workgroup: parameters and mirrored neighbour weights ----
     // w : this cell's weights (forward recompute)
     // v : V[t][c] = W[26-t, c + off_t], what the neighbour at c + off_t multiplies cell c by
     // nw: gradient of that same neighbour weight; it is the product of this cell's x and the
@@ -492,15 +416,9 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
 #pragma unroll
     for (int t = 0; t < 27; ++t) {
         load_cells<CPT>(weight + t * cells + pl.gc, w[t]);
-        const int a = t / 9, b = (t / 3) % 3, cc = t % 3;
-        const int ni = pl.i + a - 1, nj = pl.j + b - 1;
-        const bool row_in = ni >= 0 && ni < BS && nj >= 0 && nj < BS;
 #pragma unroll
         for (int c = 0; c < CPT; ++c) {
-            const int nk = pl.kt * CPT + c + cc - 1;
-            const bool in = row_in && nk >= 0 && nk < BS;
-            v[t][c] = in ? weight[(26 - t) * cells + pl.gc + c + ((a - 1) * N + (b - 1)) * K + (cc - 1)]
-                         : 0.f;
+            v[t][c] = in_block(t, c) ? weight[neighbour_weight(t, c)] : 0.f;
             nw[t][c] = 0.f;
         }
     }
@@ -509,98 +427,53 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
 #pragma unroll
     for (int c = 0; c < CPT; ++c) db[c] = dr[c] = 0.f;
 
-    {
-        constexpr int NP = TL::NH * TL::NPAIR, NE = (NP + NT - 1) / NT;
-        const int *words = pair_words<BS>();
-        int word[NE];
-        float wt[NE];
-#pragma unroll
-        for (int n = 0; n < NE; ++n) {
-            const int e = threadIdx.x + n * NT;
-            word[n] = e < NP ? words[e] : 0;
-        }
-#pragma unroll
-        for (int n = 0; n < NE; ++n)  // all gathers in flight together
-            wt[n] = word[n] < 0 ? weight[((word[n] >> 16) & 31) * cells +
-                                         pair_source_cell<TL>(word[n], pl.p0, pl.q0, pl.r0, N, K)]
-                                : 0.f;
-#pragma unroll
-        for (int n = 0; n < NE; ++n) {
-            const int e = threadIdx.x + n * NT;
-            // invalid pairs read window entry 0, a halo corner of the delta window: zero
-            if (e < NP) tab[e] = make_float2(wt[n], __int_as_float(word[n] & 0xffff));
-        }
-    }
-    // the halo entries this thread serves for every batch element, and the gradients of the
-    // weights whose tap reads them: x on the halo is frozen, so these need only D = sum_i delta_i
-    int hoff[NHPT];
-    float hw[NHPT][TL::NPAIR];
-#pragma unroll
-    for (int k = 0; k < NHPT; ++k) {
-        const int hh = pl.lane + k * TL::TPS;
-        int wi = 0, wj = 0, wk = 0;
-        if (hh < TL::NH) halo_coords<TL>(hh, wi, wj, wk);
-        hoff[k] = wi * TL::PS + wj * TL::RS + wk;
-#pragma unroll
-        for (int q = 0; q < TL::NPAIR; ++q) hw[k][q] = 0.f;
-    }
     // delta windows: the halo stays zero for the whole kernel
     for (int idx = pl.lane; idx < 2 * TL::WIN; idx += TL::TPS) dwin[idx] = 0.f;
     wait_global_loads();
+    // Add-in-place mode: slot 0's accumulators start from what the gradient buffers hold and
+    // are stored at the end like in the overwrite mode.  Requested here, behind the set-up
+    // wait, the old values arrive while the first element is recomputed.
+    if (param_mode == kParamAddExclusive && pl.slot == 0) {
+#pragma unroll
+        for (int t = 0; t < 27; ++t)
+#pragma unroll
+            for (int c = 0; c < CPT; ++c)
+                if (in_block(t, c)) nw[t][c] = dweight[neighbour_weight(t, c)];
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) {
+            db[c] = dbias[pl.gc + c];
+            dr[c] = dscale[pl.gc + c];
+        }
+    }
 
     const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
-    float pre[Fetch<TL>::RPT][TL::S], g[CPT];
+    float pre[Fetch<TL>::RPT][Fetch<TL>::HL], g[CPT];
     if (s0 + pl.slot < s1) {
         fx.fetch(x + (s0 + pl.slot) * cells, pre);
         load_cells<CPT>(dy + (s0 + pl.slot) * cells + pl.gc, g);
     }
-    // Per element: commit its window, barrier, [halo pass and stores of the PREVIOUS element],
-    // recompute, reverse sweep, write D = sum_i delta_i into delta copy 1, commit the next
-    // window.  Deferring the halo pass past the next barrier saves a barrier per element, lets
-    // its dependent LDS look-ups overlap the first stencil loads of the next element, and keeps
-    // the stores away from the wait on the prefetched window (loads and stores share one
-    // in-order counter).
-    float g_done[CPT], xh[NHPT], xh_done[NHPT];
+    // Per element: commit its window, barrier, [stores of the PREVIOUS element], recompute,
+    // reverse sweep, commit the next window.  The stores are issued one element late, away from
+    // the wait on the prefetched window (loads and stores share one in-order counter).  Besides
+    // the gradient of its own cells a thread leaves D = sum_i delta_i of them: what the cells
+    // of neighbouring blocks and the weights of taps that read the frozen halo receive depends
+    // on the iterations only through D, and a second kernel (step_bwd_cross) works it out.
+    float g_done[CPT], d_done[CPT];
     int done_s = -1;
-    auto finish_done = [&]() {  // call only after a barrier that follows the D write
+    auto finish_done = [&]() {
         if (done_s < 0) return;
-        float *hs = halo_out + ((long)done_s * nblk + blk) * TL::NH;
-#pragma unroll
-        for (int k = 0; k < NHPT; ++k) {
-            const int hh = pl.lane + k * TL::TPS;
-            if (hh < TL::NH) {
-                float2 ent[TL::NPAIR];
-#pragma unroll
-                for (int q = 0; q < TL::NPAIR; ++q) ent[q] = tab[hh * TL::NPAIR + q];
-                float acc = 0.f;
-#pragma unroll
-                for (int q = 0; q < TL::NPAIR; ++q) {
-                    const float d = dwin[TL::WIN + __float_as_int(ent[q].y)];
-                    acc = fmaf(ent[q].x, d, acc);
-                    hw[k][q] = fmaf(xh_done[k], d, hw[k][q]);
-                }
-                hs[hh] = acc;
-            }
-        }
-        if (dx_accumulate) add_cells<CPT>(dx + done_s * cells + pl.gc, g_done);
-        else store_cells<CPT>(dx + done_s * cells + pl.gc, g_done);
+        const long o = (long)done_s * cells + pl.gc;
+        store_cells<CPT>(dsum_out + o, d_done);
+        if (dx_accumulate) add_cells<CPT>(dx + o, g_done);
+        else store_cells<CPT>(dx + o, g_done);
         done_s = -1;
     };
     if (s0 + pl.slot < s1) fx.commit(win, pre);
-#ifdef EXP_TIMING
-    long t_acc[5] = {0, 0, 0, 0, 0};
-    long t_prev = clock64();
-#define TICK(i) { long t_now = clock64(); t_acc[i] += t_now - t_prev; t_prev = t_now; }
-#else
-#define TICK(i)
-#endif
     for (int sb = s0; sb < s1; sb += NSLOT) {
         const int s = sb + pl.slot;
         const bool active = s < s1;  // a slot past the end idles through the barriers
-        lds_barrier();               // this element's window and the previous element's D
-        TICK(0)
+        lds_barrier();               // this element's window
         finish_done();
-        TICK(1)
         float gnext[CPT];
         if (s + NSLOT < s1) {
             fx.fetch(x + (s + NSLOT) * cells, pre);
@@ -610,9 +483,6 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
         if (active) {
 #pragma unroll
             for (int c = 0; c < CPT; ++c) cur[c] = win[pl.own + c];
-            // x on the halo (identical in both window copies, frozen for the whole element)
-#pragma unroll
-            for (int k = 0; k < NHPT; ++k) xh[k] = win[hoff[k]];
         }
 
         // ---- forward recompute, remembering x_i and u_i of the owned cells ----
@@ -634,7 +504,6 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
             if (it + 1 < inner) lds_barrier();
         }
 
-        TICK(2)
         // ---- reverse sweep: delta window copy (it & 1) holds delta_it ----
         float dsum[CPT], xi[CPT];
 #pragma unroll
@@ -671,34 +540,18 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
             }
         }
 
-        TICK(3)
-        // ---- cells of the neighbouring blocks need only D = sum_i delta_i (the halo is frozen);
-        // D goes to delta copy 1: the last iteration (it = 0) used copy 0 and the readers of
-        // copy 1 (it = 1) are past the barrier of it = 0.  The pass itself runs after the next
-        // barrier (finish_done).
         if (inner == 0) lds_barrier();  // no barrier since the top: others may still read LDS
-        if (active) {
-#pragma unroll
-            for (int c = 0; c < CPT; ++c) dwin[TL::WIN + pl.own + c] = dsum[c];
-        }
         done_s = active ? s : -1;
 #pragma unroll
         for (int c = 0; c < CPT; ++c) {
             g_done[c] = g[c];
+            d_done[c] = dsum[c];
             g[c] = gnext[c];
         }
-#pragma unroll
-        for (int k = 0; k < NHPT; ++k) xh_done[k] = xh[k];
         // the x windows are free (the reverse sweep does not read them): commit the next one
         if (s + NSLOT < s1) fx.commit(win, pre);
-        TICK(4)
     }
-    lds_barrier();
     finish_done();
-#ifdef EXP_TIMING
-    if (threadIdx.x == 0)
-        for (int i = 0; i < 5; ++i) halo_out[blk * 8 + i] = (float)t_acc[i];
-#endif
 
     // ---- parameter gradients: reduce across slots through LDS, then commit ----
     if (NSLOT > 1) {
@@ -721,89 +574,169 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_fast(
             reduce(db[c]);
             reduce(dr[c]);
         }
-#pragma unroll
-        for (int k = 0; k < NHPT; ++k)
-#pragma unroll
-            for (int q = 0; q < TL::NPAIR; ++q) reduce(hw[k][q]);
         if (pl.slot != 0) return;
     }
+    commit_grads<27, CPT>(dweight, nw, param_mode, neighbour_weight, in_block);
+    float one[1][CPT];
+    auto own_cell = [&](int, int c) { return pl.gc + c; };
+    auto always = [](int, int) { return true; };
+#pragma unroll
+    for (int c = 0; c < CPT; ++c) one[0][c] = db[c];
+    commit_grads<1, CPT>(dbias, one, param_mode, own_cell, always);
+#pragma unroll
+    for (int c = 0; c < CPT; ++c) one[0][c] = dr[c];
+    commit_grads<1, CPT>(dscale, one, param_mode, own_cell, always);
+}
+
+// ---- backward, second kernel: everything that crosses a block boundary ----------------------
+// The window halo is frozen during the inner iterations, so both the gradient that the cells of
+// NEIGHBOURING blocks receive and the gradient of a weight whose tap reads a halo entry depend
+// on the iterations only through D = sum_i delta_i, which step_bwd_fast leaves in `dsum`:
+//   dx[c]    += sum over taps t with c + off_t in another block of W[26-t, c + off_t] * D[c + off_t]
+//   dW[t, c] += D[c] * x[c + off_t]          for the taps t whose c + off_t lies outside c's block
+// Same mapping as the main kernel (a slot per (block, batch element), CPT cells per thread,
+// weights and gradient accumulators in registers) with the x window and the D window of the
+// element in LDS, both with their REAL halo this time: the neighbouring blocks' values, zero
+// outside the grid.  One stencil-shaped pass per element; no atomics, fixed order.  Two stages
+// of windows alternate, which leaves one barrier per element.
+constexpr int kCrossDepth = 4;  // neighbour rows requested ahead of the arithmetic
+
+template <int BS, int CPT, int NSLOT>
+__global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_cross(
+    const float *__restrict__ weight, const float *__restrict__ x, const float *__restrict__ dsum,
+    float *__restrict__ dweight, float *__restrict__ dx, int B, int M, int N, int K, int nblk,
+    int nchunk, int chunk_len, int param_mode) {
+    using TL = Tile<BS, CPT>;
+    constexpr int STAGE = 2 * TL::WIN;  // [x window | D window]
+    __shared__ __attribute__((aligned(16))) float lds[NSLOT * 2 * STAGE];
+
+    int blk, chunk;
+    if (!split_block_id(blockIdx.x, nblk, nchunk, blk, chunk)) return;  // grid padding
+    const Place<TL, CPT, NSLOT> pl(threadIdx.x, blk, N, K);
+    const Fetch<TL> fx(pl.lane, pl.p0, pl.q0, pl.r0, M, N, K);
+    float *stages = lds + pl.slot * (2 * STAGE);
+    const long cells = (long)M * N * K;
+
+    auto leaves_block = [&](int t, int c) {
+        const int ni = pl.i + t / 9 - 1, nj = pl.j + (t / 3) % 3 - 1, nk = pl.kt * CPT + c + t % 3 - 1;
+        return !(ni >= 0 && ni < BS && nj >= 0 && nj < BS && nk >= 0 && nk < BS);
+    };
+    // vx: V[t][c] = W[26-t, c + off_t] where the neighbour lies in ANOTHER block of the grid
+    //     (the complement of the main kernel's v); cw: gradient of this cell's own tap t.
+    float vx[27][CPT], cw[27][CPT];
+    bool any_cross = false;
 #pragma unroll
     for (int t = 0; t < 27; ++t) {
         const int a = t / 9, b = (t / 3) % 3, cc = t % 3;
         const int ni = pl.i + a - 1, nj = pl.j + b - 1;
         const bool row_in = ni >= 0 && ni < BS && nj >= 0 && nj < BS;
+        const int gi = pl.p0 + ni, gj = pl.q0 + nj;
+        const bool row_grid = gi >= 0 && gi < M && gj >= 0 && gj < N;
 #pragma unroll
         for (int c = 0; c < CPT; ++c) {
-            const int nk = pl.kt * CPT + c + cc - 1;
-            if (row_in && nk >= 0 && nk < BS)
-                commit_grad(dweight + (26 - t) * cells + pl.gc + c + ((a - 1) * N + (b - 1)) * K + (cc - 1),
-                            nw[t][c], param_mode);
+            const int nk = pl.kt * CPT + c + cc - 1, gk = pl.r0 + nk;
+            const bool leaves = !(row_in && nk >= 0 && nk < BS);
+            const bool cross = leaves && row_grid && gk >= 0 && gk < K;
+            vx[t][c] = cross ? weight[(26 - t) * cells + pl.gc + c + ((a - 1) * N + (b - 1)) * K + (cc - 1)]
+                             : 0.f;
+            cw[t][c] = 0.f;
+            any_cross = any_cross || cross;
         }
     }
+    wait_global_loads();
+    // add-in-place mode: slot 0's accumulators start from what the gradient buffer holds
+    if (param_mode == kParamAddExclusive && pl.slot == 0) {
 #pragma unroll
-    for (int k = 0; k < NHPT; ++k) {
-        const int hh = pl.lane + k * TL::TPS;
-        if (hh < TL::NH) {
+        for (int t = 0; t < 27; ++t)
 #pragma unroll
-            for (int q = 0; q < TL::NPAIR; ++q) {
-                const int word = pair_words<BS>()[hh * TL::NPAIR + q];
-                if (word < 0)
-                    commit_grad(dweight + ((word >> 16) & 31) * cells +
-                                    pair_source_cell<TL>(word, pl.p0, pl.q0, pl.r0, N, K),
-                                hw[k][q], param_mode);
-            }
-        }
+            for (int c = 0; c < CPT; ++c)
+                if (leaves_block(t, c)) cw[t][c] = dweight[t * cells + pl.gc + c];
     }
-#pragma unroll
-    for (int c = 0; c < CPT; ++c) {
-        commit_grad(dbias + pl.gc + c, db[c], param_mode);
-        commit_grad(dscale + pl.gc + c, dr[c], param_mode);
-    }
-}
 
-// dx[cell] += the halo contributions of the (up to 7) neighbouring blocks whose window contains
-// the cell, added in a fixed order.  One thread owns one K-row of one block (bs cells): whether
-// a neighbour in i or j reaches the row is decided once per row, and those contributions are
-// bs consecutive floats of the neighbour's compacted halo; only the two end cells of the row
-// also see neighbours in k.  blockIdx.y = sample.
-template <int BS>
-__global__ __launch_bounds__(256) void halo_gather(const float *__restrict__ halo,
-                                                   float *__restrict__ dx, int M, int N, int K,
-                                                   int nblk, int rows_per_sample) {
-    using TL = Tile<BS, 1>;
-    const int row = blockIdx.x * blockDim.x + threadIdx.x;  // (gi, gj, bk), bk fastest
-    if (row >= rows_per_sample) return;
-    const int kb = K / BS, nb = N / BS, mb = M / BS;
-    const int bk = row % kb;
-    const int gj = (row / kb) % N;
-    const int gi = row / (kb * N);
-    const int li = gi % BS, lj = gj % BS, bi = gi / BS, bj = gj / BS;
-    const int di_lo = (li == 0 && bi > 0) ? -1 : 0, di_hi = (li == BS - 1 && bi < mb - 1) ? 1 : 0;
-    const int dj_lo = (lj == 0 && bj > 0) ? -1 : 0, dj_hi = (lj == BS - 1 && bj < nb - 1) ? 1 : 0;
-    const float *hs = halo + (size_t)blockIdx.y * nblk * TL::NH;
-    float acc[BS];
-#pragma unroll
-    for (int c = 0; c < BS; ++c) acc[c] = 0.f;
-    for (int di = di_lo; di <= di_hi; ++di)
-        for (int dj = dj_lo; dj <= dj_hi; ++dj) {
-            const int wi = li + 1 - di * BS, wj = lj + 1 - dj * BS;  // row in the neighbour's window
-            const int other = ((bi + di) * nb + (bj + dj)) * kb + bk;
-            if (di != 0 || dj != 0) {  // the neighbour's halo holds the whole row, contiguously
-                const float *src = hs + (size_t)other * TL::NH + halo_index<TL>(wi, wj, 1);
-#pragma unroll
-                for (int c = 0; c < BS; ++c) acc[c] += src[c];
-            }
-            // neighbours one block further along k reach only the row's end cells
-            if (bk > 0) acc[0] += hs[(size_t)(other - 1) * TL::NH + halo_index<TL>(wi, wj, BS + 1)];
-            if (bk < kb - 1) acc[BS - 1] += hs[(size_t)(other + 1) * TL::NH + halo_index<TL>(wi, wj, 0)];
+    // Windows are fetched TWO elements ahead (two register buffers, used alternately): with one
+    // stencil pass per element there is too little arithmetic to cover a trip to memory.
+    const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
+    using Buf = float[Fetch<TL>::RPT][Fetch<TL>::HL];
+    Buf ax, ad, bx, bd;
+    auto fetch_into = [&](int s, Buf &px, Buf &pd) {
+        if (s < s1) {
+            fx.fetch(x + (long)s * cells, px);
+            fx.fetch(dsum + (long)s * cells, pd);
         }
-    float *out = dx + ((size_t)blockIdx.y * M * N + (size_t)gi * N + gj) * K + bk * BS;
+    };
+    auto commit_from = [&](int s, int st, const Buf &px, const Buf &pd) {
+        if (s < s1) {
+            fx.template commit<1>(stages + st * STAGE, px);
+            fx.template commit<1>(stages + st * STAGE + TL::WIN, pd);
+        }
+    };
+    // One element: stage `st` holds it, `px/pd` hold the next one (in flight or arrived), the
+    // other buffer pair `qx/qd` is free and receives the element after that.
+    auto element = [&](int s, int st, const Buf &px, const Buf &pd, Buf &qx, Buf &qd) {
+        const bool active = s < s1;
+        lds_barrier();  // stage `st` is complete; every reader of the other stage is done
+        float gx[CPT];  // dx of the owned cells so far (their own block's part)
+        float *out = dx + (long)s * cells + pl.gc;
+        if (active && any_cross) load_cells<CPT>(out, gx);  // before the prefetch: it is awaited first
+        fetch_into(s + 2 * NSLOT, qx, qd);
+        if (active) {
+            const float *xw = stages + st * STAGE, *dw = xw + TL::WIN;
+            float dc[CPT], g[CPT];
 #pragma unroll
-    for (int q = 0; q < BS / 4; ++q) {
-        float4 o = *reinterpret_cast<float4 *>(out + 4 * q);
-        o.x += acc[4 * q]; o.y += acc[4 * q + 1]; o.z += acc[4 * q + 2]; o.w += acc[4 * q + 3];
-        *reinterpret_cast<float4 *>(out + 4 * q) = o;
+            for (int c = 0; c < CPT; ++c) {
+                dc[c] = dw[pl.own + c];
+                g[c] = 0.f;
+            }
+            for_each_row<TL, CPT, kCrossDepth>(dw + pl.row00, [&](int r, const float (&dv)[CPT + 2]) {
+#pragma unroll
+                for (int cc = 0; cc < 3; ++cc)
+#pragma unroll
+                    for (int c = 0; c < CPT; ++c) g[c] = fmaf(vx[r * 3 + cc][c], dv[c + cc], g[c]);
+            });
+            for_each_row<TL, CPT, kCrossDepth>(xw + pl.row00, [&](int r, const float (&xv)[CPT + 2]) {
+#pragma unroll
+                for (int cc = 0; cc < 3; ++cc)
+#pragma unroll
+                    for (int c = 0; c < CPT; ++c)
+                        cw[r * 3 + cc][c] = fmaf(dc[c], xv[c + cc], cw[r * 3 + cc][c]);
+            });
+            if (any_cross) {
+#pragma unroll
+                for (int c = 0; c < CPT; ++c) gx[c] += g[c];
+                store_cells<CPT>(out, gx);
+            }
+        }
+        commit_from(s + NSLOT, st ^ 1, px, pd);
+    };
+    fetch_into(s0 + pl.slot, ax, ad);
+    fetch_into(s0 + pl.slot + NSLOT, bx, bd);
+    commit_from(s0 + pl.slot, 0, ax, ad);
+    for (int sb = s0; sb < s1; sb += 2 * NSLOT) {
+        element(sb + pl.slot, 0, bx, bd, ax, ad);
+        element(sb + pl.slot + NSLOT, 1, ax, ad, bx, bd);  // may lie past the end: idles
     }
+
+    if (NSLOT > 1) {
+        float *red = lds;  // NSLOT * TPS floats, reused value by value
+#pragma unroll
+        for (int t = 0; t < 27; ++t)
+#pragma unroll
+            for (int c = 0; c < CPT; ++c) {
+                lds_barrier();
+                red[pl.slot * TL::TPS + pl.lane] = cw[t][c];
+                lds_barrier();
+                if (pl.slot == 0) {
+#pragma unroll
+                    for (int q = 1; q < NSLOT; ++q) cw[t][c] += red[q * TL::TPS + pl.lane];
+                }
+            }
+        if (pl.slot != 0) return;
+    }
+    // every tap that leaves the block is committed, also where it reads the zero padding outside
+    // the grid (its gradient is exactly zero and a store-mode caller expects every entry written)
+    commit_grads<27, CPT>(
+        dweight, cw, param_mode, [&](int t, int c) { return t * cells + pl.gc + c; },
+        leaves_block);
 }
 
 __global__ void fill_zero_f32(float *p, long n) {
@@ -875,6 +808,10 @@ template <int BS, int CPT, int NSLOT, int ACT> int launch_fwd(const StepArgs &a,
 
 constexpr size_t kMaxLds = 160 * 1024;
 
+// the cross-block kernel's own shapes (it shares the main kernel's blocks and batch chunks)
+constexpr int kCrossCpt8 = 2, kCrossSlots8 = 1;  // bs=8: 256 threads
+constexpr int kCrossCpt4 = 1, kCrossSlots4 = 4;  // bs=4: four one-wave slots
+
 template <int BS, int CPT, int NSLOT, int ACT> int launch_bwd(const StepArgs &a, hipStream_t st) {
     using TL = Tile<BS, CPT>;
     const long cells = (long)a.M * a.N * a.K;
@@ -913,29 +850,20 @@ template <int BS, int CPT, int NSLOT, int ACT> int launch_bwd(const StepArgs &a,
         if (int rc = fill_zero((float *)a.dscale, cells, st)) return rc;
     }
     const int dx_accumulate = (a.flags & GRIDNET_OVERWRITE_DX) ? 0 : 1;
-    {   // the pair table of this block size, once per device (idempotent, stream-ordered)
-        static bool built[64] = {false};
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess) dev = -1;
-        if (dev >= 0 && dev < 64 && !built[dev]) {
-            constexpr int NP = Tile<BS, 1>::NH * Tile<BS, 1>::NPAIR;
-            hipLaunchKernelGGL((build_pair_words<BS>), dim3((NP + 255) / 256), dim3(256), 0, st);
-            if (int rc = check_launch("build_pair_words")) return rc;
-            built[dev] = true;
-        }
-    }
     hipLaunchKernelGGL(kern, dim3(padded_grid(p.nblk, p.nchunk)), dim3(TL::TPS * NSLOT), lds, st,
                        (const float *)a.weight, (const float *)a.bias, (const float *)a.scale,
                        (const float *)a.x, (const float *)a.dy, (float *)a.dweight, (float *)a.dbias,
                        (float *)a.dscale, (float *)a.dx, (float *)a.workspace, a.B, a.M, a.N, a.K,
                        a.inner, p.nblk, p.nchunk, p.chunk_len, param_mode, dx_accumulate);
     if (int rc = check_launch("step_bwd_fast")) return rc;
-    if (nblk > 1) {
-        const int rows = a.M * a.N * (a.K / BS);
-        hipLaunchKernelGGL((halo_gather<BS>), dim3((rows + 255) / 256, a.B), dim3(256), 0, st,
-                           (const float *)a.workspace, (float *)a.dx, a.M, a.N, a.K, nblk, rows);
-        if (int rc = check_launch("halo_gather")) return rc;
-    }
+    // same blocks, same batch chunks, same way of committing parameter gradients (the two
+    // kernels write disjoint entries of dweight)
+    constexpr int XCPT = BS == 8 ? kCrossCpt8 : kCrossCpt4, XSLOT = BS == 8 ? kCrossSlots8 : kCrossSlots4;
+    hipLaunchKernelGGL((step_bwd_cross<BS, XCPT, XSLOT>), dim3(padded_grid(p.nblk, p.nchunk)),
+                       dim3(Tile<BS, XCPT>::TPS * XSLOT), 0, st, (const float *)a.weight,
+                       (const float *)a.x, (const float *)a.workspace, (float *)a.dweight,
+                       (float *)a.dx, a.B, a.M, a.N, a.K, p.nblk, p.nchunk, p.chunk_len, param_mode);
+    if (int rc = check_launch("step_bwd_cross")) return rc;
     return GRIDNET_OK;
 }
 
@@ -978,10 +906,8 @@ bool step_fast_supports(const StepArgs &a, bool backward) {
 }
 
 size_t step_fast_backward_workspace(const StepArgs &a) {
-    const int bs = a.block_size;
-    const size_t nblk = (size_t)(a.M / bs) * (a.N / bs) * (a.K / bs);
-    const size_t nh = bs == 8 ? Tile<8, 1>::NH : Tile<4, 1>::NH;
-    return (size_t)a.B * nblk * nh * sizeof(float);
+    // D = sum_i delta_i of every cell, handed from step_bwd_fast to step_bwd_cross
+    return (size_t)a.B * a.M * a.N * a.K * sizeof(float);
 }
 
 int step_forward_fast(const StepArgs &a, hipStream_t st) { return dispatch<false>(a, st); }
