@@ -163,10 +163,11 @@ template <typename TL, int CPT, int NSLOT> struct Place {
 // entry plus bs/2 cells of the block; the cells are contiguous and 16-byte (bs=8) or 8-byte
 // (bs=4) aligned in the grid and come in as one vector.  End entries belong to the
 // neighbouring blocks, or lie outside the grid and read as zero (gridnet/backend_torch.py:63).
-template <typename TL> struct Fetch {
+template <typename TL, int NT = TL::TPS> struct Fetch {  // NT: threads of a slot
     static constexpr int S = TL::S, BS = TL::S - 2, HL = S / 2, HC = BS / 2;
     static constexpr int NHALF = 2 * S * S;
-    static constexpr int RPT = (NHALF + TL::TPS - 1) / TL::TPS;  // half rows per thread
+    static constexpr int RPT = (NHALF + NT - 1) / NT;  // half rows per thread
+    using Buf = float[RPT][HL];
     int goff[RPT];   // grid offset (within a sample) of the half row's first block cell; rows
                      // outside the grid point at a valid address and are zeroed when committed
     int loff[RPT];   // LDS offset of the half row's first entry, -1: none for this thread
@@ -177,7 +178,7 @@ template <typename TL> struct Fetch {
     __device__ __forceinline__ Fetch(int lane, int p0, int q0, int r0, int M, int N, int K) {
 #pragma unroll
         for (int e = 0; e < RPT; ++e) {
-            const int id = lane + e * TL::TPS;
+            const int id = lane + e * NT;
             const int half = id & 1, row = id >> 1;
             const int wj = row % S, wi = row / S;
             const int gi = p0 + wi - 1, gj = q0 + wj - 1;
@@ -194,7 +195,7 @@ template <typename TL> struct Fetch {
         }
     }
     // Unconditional loads (no branches, no register initialisation in front of them).
-    __device__ __forceinline__ void fetch(const float *xs, float (&v)[RPT][HL]) const {
+    __device__ __forceinline__ void fetch(const float *xs, Buf &v) const {
 #pragma unroll
         for (int e = 0; e < RPT; ++e) {
             const float *p = xs + goff[e];
@@ -210,7 +211,7 @@ template <typename TL> struct Fetch {
     // Both window copies receive every entry (the halo must be in both; the block itself is
     // overwritten by the iterations anyway).
     template <int COPIES = 2>
-    __device__ __forceinline__ void commit(float *win, const float (&v)[RPT][HL]) const {
+    __device__ __forceinline__ void commit(float *win, const Buf &v) const {
 #pragma unroll
         for (int e = 0; e < RPT; ++e)
             if (loff[e] >= 0) {
@@ -224,6 +225,63 @@ template <typename TL> struct Fetch {
                     for (int q = 0; q < HC; ++q) row[q + (hi[e] ? 0 : 1)] = ok[e] ? v[e][q] : 0.f;
                 }
             }
+    }
+};
+
+// The same job for a kernel whose time goes into the memory pipeline rather than arithmetic
+// (step_bwd_cross): every window row is read as bs/4 + 2 aligned 16-byte vectors by ADJACENT
+// lanes -- the vector before the block (only its last float is an entry of the window), the
+// block's own vectors, the vector after it (only its first float).  A row then costs the
+// vector cache one or two line accesses instead of one per half row plus one per end entry.
+// More registers per thread than Fetch, which is why the compute-bound kernels keep that one.
+template <typename TL, int NT> struct FetchLines {
+    static constexpr int S = TL::S, BS = TL::S - 2, NQ = BS / 4 + 2;
+    static constexpr int NVEC = S * S * NQ;
+    static constexpr int RPT = (NVEC + NT - 1) / NT;  // vectors per thread
+    using Buf = float[RPT][4];
+    int goff[RPT];   // grid offset (within a sample) of the vector
+    int meta[RPT];   // bits 0..11: LDS offset of the first window entry the vector fills;
+                     // bits 12..13: 0 all four floats are entries, 1 only the last, 2 only the
+                     // first, 3 nothing (no vector for this thread); bit 14: inside the grid
+    __device__ __forceinline__ FetchLines(int lane, int p0, int q0, int r0, int M, int N, int K) {
+        static_assert(TL::WIN < 4096, "window offsets must fit 12 bits");
+#pragma unroll
+        for (int e = 0; e < RPT; ++e) {
+            const int id = lane + e * NT;
+            const int qd = id % NQ, row = id / NQ;
+            const int wj = row % S, wi = row / S;
+            const int gi = p0 + wi - 1, gj = q0 + wj - 1, col = r0 + 4 * (qd - 1);
+            const bool have = id < NVEC;
+            const bool ok = have && gi >= 0 && gi < M && gj >= 0 && gj < N && col >= 0 && col < K;
+            const int kind = !have ? 3 : qd == 0 ? 1 : qd == NQ - 1 ? 2 : 0;
+            const int wk = qd == 0 ? 0 : qd == NQ - 1 ? S - 1 : 1 + 4 * (qd - 1);
+            meta[e] = (have ? wi * TL::PS + wj * TL::RS + wk : 0) | (kind << 12) | (ok ? 1 << 14 : 0);
+            // anything outside the grid (and threads without a vector) reads the start of row
+            // (0, 0) of the block's own columns: always in bounds
+            goff[e] = ok ? (gi * N + gj) * K + col : r0;
+        }
+    }
+    __device__ __forceinline__ void fetch(const float *xs, Buf &v) const {
+#pragma unroll
+        for (int e = 0; e < RPT; ++e) load_cells<4>(xs + goff[e], v[e]);
+    }
+    template <int COPIES = 2> __device__ __forceinline__ void commit(float *win, const Buf &v) const {
+#pragma unroll
+        for (int e = 0; e < RPT; ++e) {
+            const int kind = (meta[e] >> 12) & 3;
+            const bool ok = (meta[e] >> 14) & 1;
+            float *to = win + (meta[e] & 0xfff);
+            if (kind == 0) {
+#pragma unroll
+                for (int copy = 0; copy < COPIES; ++copy)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) to[copy * TL::WIN + q] = ok ? v[e][q] : 0.f;
+            } else if (kind != 3) {
+                const float end = ok ? (kind == 1 ? v[e][3] : v[e][0]) : 0.f;
+#pragma unroll
+                for (int copy = 0; copy < COPIES; ++copy) to[copy * TL::WIN] = end;
+            }
+        }
     }
 };
 
@@ -303,7 +361,7 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_fwd_fast(
     wait_global_loads();
 
     const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
-    float pre[Fetch<TL>::RPT][Fetch<TL>::HL];
+    typename Fetch<TL>::Buf pre;
     if (s0 + pl.slot < s1) fx.fetch(x + (s0 + pl.slot) * cells, pre);
     // The result of an element is stored one element late, after the next window has been
     // committed: the wait for the prefetched window would otherwise also wait for a store that
@@ -447,7 +505,8 @@ void step_bwd_fast(
     }
 
     const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
-    float pre[Fetch<TL>::RPT][Fetch<TL>::HL], g[CPT];
+    typename Fetch<TL>::Buf pre;
+    float g[CPT];
     if (s0 + pl.slot < s1) {
         fx.fetch(x + (s0 + pl.slot) * cells, pre);
         load_cells<CPT>(dy + (s0 + pl.slot) * cells + pl.gc, g);
@@ -591,152 +650,205 @@ void step_bwd_fast(
 // ---- backward, second kernel: everything that crosses a block boundary ----------------------
 // The window halo is frozen during the inner iterations, so both the gradient that the cells of
 // NEIGHBOURING blocks receive and the gradient of a weight whose tap reads a halo entry depend
-// on the iterations only through D = sum_i delta_i, which step_bwd_fast leaves in `dsum`:
-//   dx[c]    += sum over taps t with c + off_t in another block of W[26-t, c + off_t] * D[c + off_t]
-//   dW[t, c] += D[c] * x[c + off_t]          for the taps t whose c + off_t lies outside c's block
-// Same mapping as the main kernel (a slot per (block, batch element), CPT cells per thread,
-// weights and gradient accumulators in registers) with the x window and the D window of the
-// element in LDS, both with their REAL halo this time: the neighbouring blocks' values, zero
-// outside the grid.  One stencil-shaped pass per element; no atomics, fixed order.  Two stages
-// of windows alternate, which leaves one barrier per element.
-constexpr int kCrossDepth = 4;  // neighbour rows requested ahead of the arithmetic
-
-template <int BS, int CPT, int NSLOT>
-__global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_bwd_cross(
+// on the iterations only through D = sum_i delta_i, which step_bwd_fast leaves in `dsum`.  For a
+// cell c of the block and a tap t with h = c + off_t in another block:
+//   dx[c]    += W[26-t, h] * D[h]        (h's mirrored tap reads c)
+//   dW[t, c] += D[c] * x[h]              (x[h] = 0 outside the grid)
+// Only boundary cells have such taps, and a tap leaves the block through a face: the work is
+// dealt by FACE.  A slot (one batch element of the block) is 6 faces of bs*bs threads; the
+// thread of face cell c owns the 9 taps that leave through its face, minus those that also
+// leave through a face of a lower axis (edges and corners; counted there).  So every
+// (cell, tap) pair has exactly one thread, which keeps its mirrored weight and its gradient
+// accumulator in registers for the whole batch: 9 of each.  The x window and the D window of
+// the element sit in LDS with their REAL halo (the neighbouring blocks' values, zero outside
+// the grid), two stages alternating, fetched one round ahead.  Every thread leaves what it found
+// for its cell in a small LDS slab; one round late (after the next barrier) the slot's row
+// threads add the parts of each cell to dx in a fixed order; no atomics.
+// A pass over one element is short (19 LDS reads, 18 FMAs per thread), and a block has few
+// workgroups to hide latency behind: a slot therefore takes E elements per round, so that
+// one barrier, one trip to LDS and one trip to memory serve E elements.
+template <int BS, int NSLOT, int E>
+__global__ __launch_bounds__((6 * BS * BS * NSLOT)) void step_bwd_cross(
     const float *__restrict__ weight, const float *__restrict__ x, const float *__restrict__ dsum,
     float *__restrict__ dweight, float *__restrict__ dx, int B, int M, int N, int K, int nblk,
     int nchunk, int chunk_len, int param_mode) {
-    using TL = Tile<BS, CPT>;
-    constexpr int STAGE = 2 * TL::WIN;  // [x window | D window]
-    __shared__ __attribute__((aligned(16))) float lds[NSLOT * 2 * STAGE];
+    using TL = Tile<BS, 1>;  // window geometry only
+    constexpr int FS = BS * BS, TPS = 6 * FS;
+    constexpr int PAIR = 2 * TL::WIN;              // [x window | D window] of one element
+    constexpr int STAGE = E * PAIR;                // the E elements of a round
+    constexpr int SLOT = 2 * STAGE + 2 * E * TPS;  // two stages, two slabs
+    __shared__ __attribute__((aligned(16))) float lds[NSLOT * SLOT];
 
     int blk, chunk;
     if (!split_block_id(blockIdx.x, nblk, nchunk, blk, chunk)) return;  // grid padding
-    const Place<TL, CPT, NSLOT> pl(threadIdx.x, blk, N, K);
-    const Fetch<TL> fx(pl.lane, pl.p0, pl.q0, pl.r0, M, N, K);
-    float *stages = lds + pl.slot * (2 * STAGE);
+    const int slot = NSLOT == 1 ? 0 : threadIdx.x / TPS, lane = threadIdx.x - slot * TPS;
+    const int kb = K / BS, nb = N / BS;
+    const int p0 = (blk / (kb * nb)) * BS, q0 = ((blk / kb) % nb) * BS, r0 = (blk % kb) * BS;
+    const FetchLines<TL, TPS> fx(lane, p0, q0, r0, M, N, K);
+    float *stages = lds + slot * SLOT, *slabs = stages + 2 * STAGE;
     const long cells = (long)M * N * K;
 
-    auto leaves_block = [&](int t, int c) {
-        const int ni = pl.i + t / 9 - 1, nj = pl.j + (t / 3) % 3 - 1, nk = pl.kt * CPT + c + t % 3 - 1;
-        return !(ni >= 0 && ni < BS && nj >= 0 && nj < BS && nk >= 0 && nk < BS);
-    };
-    // vx: V[t][c] = W[26-t, c + off_t] where the neighbour lies in ANOTHER block of the grid
-    //     (the complement of the main kernel's v); cw: gradient of this cell's own tap t.
-    float vx[27][CPT], cw[27][CPT];
-    bool any_cross = false;
+    // ---- which cell, which taps ----
+    const int face = lane / FS, axis = face >> 1, side = face & 1;
+    const int u = (lane % FS) / BS, v = lane % BS, fix = side ? BS - 1 : 0;
+    const int ci = axis == 0 ? fix : u;
+    const int cj = axis == 0 ? u : axis == 1 ? fix : v;
+    const int ck = axis == 2 ? fix : v;
+    const int gcell = ((p0 + ci) * N + (q0 + cj)) * K + (r0 + ck);
+    const int own = (ci + 1) * TL::PS + (cj + 1) * TL::RS + (ck + 1);
+    const int out = side ? 1 : -1;  // the face's outward direction along its axis
+    // The first bs*bs threads of the slot double as ROW threads: thread (ri, rj) adds what the
+    // faces found for the bs cells of block row (ri, rj) to dx, whole rows at a time (a row is
+    // one vector-cache line access to read and one to write; cell by cell it would be eight).
+    const bool is_row = lane < FS;
+    const int ri = lane / BS, rj = lane % BS;  // meaningful for row threads only
+    const long grow = ((long)(p0 + ri) * N + (q0 + rj)) * K + r0;
+    const bool ri_edge = ri == 0 || ri == BS - 1, rj_edge = rj == 0 || rj == BS - 1;
+
+    float vx[9], cw[9];
+    int hoff[9];
+    bool mine[9];
 #pragma unroll
-    for (int t = 0; t < 27; ++t) {
-        const int a = t / 9, b = (t / 3) % 3, cc = t % 3;
-        const int ni = pl.i + a - 1, nj = pl.j + b - 1;
-        const bool row_in = ni >= 0 && ni < BS && nj >= 0 && nj < BS;
-        const int gi = pl.p0 + ni, gj = pl.q0 + nj;
-        const bool row_grid = gi >= 0 && gi < M && gj >= 0 && gj < N;
-#pragma unroll
-        for (int c = 0; c < CPT; ++c) {
-            const int nk = pl.kt * CPT + c + cc - 1, gk = pl.r0 + nk;
-            const bool leaves = !(row_in && nk >= 0 && nk < BS);
-            const bool cross = leaves && row_grid && gk >= 0 && gk < K;
-            vx[t][c] = cross ? weight[(26 - t) * cells + pl.gc + c + ((a - 1) * N + (b - 1)) * K + (cc - 1)]
-                             : 0.f;
-            cw[t][c] = 0.f;
-            any_cross = any_cross || cross;
-        }
+    for (int pq = 0; pq < 9; ++pq) {
+        const int dp = pq / 3 - 1, dq = pq % 3 - 1;  // steps along the two in-face axes
+        const int di = axis == 0 ? out : dp;
+        const int dj = axis == 0 ? dp : axis == 1 ? out : dq;
+        const int dk = axis == 2 ? out : dq;
+        const int t = (di + 1) * 9 + (dj + 1) * 3 + (dk + 1);
+        // also leaving through a face of a lower axis: that face's thread has the pair
+        const bool lower = (axis >= 1 && ((di < 0 && ci == 0) || (di > 0 && ci == BS - 1))) ||
+                           (axis == 2 && ((dj < 0 && cj == 0) || (dj > 0 && cj == BS - 1)));
+        const int gi = p0 + ci + di, gj = q0 + cj + dj, gk = r0 + ck + dk;
+        const bool in_grid = gi >= 0 && gi < M && gj >= 0 && gj < N && gk >= 0 && gk < K;
+        mine[pq] = !lower;
+        hoff[pq] = own + di * TL::PS + dj * TL::RS + dk;
+        const long hcell = gcell + (long)(di * N + dj) * K + dk;
+        vx[pq] = (mine[pq] && in_grid) ? weight[(26 - t) * cells + hcell] : 0.f;
+        // add-in-place mode: slot 0's accumulators start from what the gradient buffer holds
+        cw[pq] = (mine[pq] && param_mode == kParamAddExclusive && slot == 0)
+                     ? dweight[t * cells + gcell]
+                     : 0.f;
     }
     wait_global_loads();
-    // add-in-place mode: slot 0's accumulators start from what the gradient buffer holds
-    if (param_mode == kParamAddExclusive && pl.slot == 0) {
-#pragma unroll
-        for (int t = 0; t < 27; ++t)
-#pragma unroll
-            for (int c = 0; c < CPT; ++c)
-                if (leaves_block(t, c)) cw[t][c] = dweight[t * cells + pl.gc + c];
-    }
 
-    // Windows are fetched TWO elements ahead (two register buffers, used alternately): with one
-    // stencil pass per element there is too little arithmetic to cover a trip to memory.
     const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
-    using Buf = float[Fetch<TL>::RPT][Fetch<TL>::HL];
-    Buf ax, ad, bx, bd;
-    auto fetch_into = [&](int s, Buf &px, Buf &pd) {
-        if (s < s1) {
-            fx.fetch(x + (long)s * cells, px);
-            fx.fetch(dsum + (long)s * cells, pd);
-        }
-    };
-    auto commit_from = [&](int s, int st, const Buf &px, const Buf &pd) {
-        if (s < s1) {
-            fx.template commit<1>(stages + st * STAGE, px);
-            fx.template commit<1>(stages + st * STAGE + TL::WIN, pd);
-        }
-    };
-    // One element: stage `st` holds it, `px/pd` hold the next one (in flight or arrived), the
-    // other buffer pair `qx/qd` is free and receives the element after that.
-    auto element = [&](int s, int st, const Buf &px, const Buf &pd, Buf &qx, Buf &qd) {
-        const bool active = s < s1;
-        lds_barrier();  // stage `st` is complete; every reader of the other stage is done
-        float gx[CPT];  // dx of the owned cells so far (their own block's part)
-        float *out = dx + (long)s * cells + pl.gc;
-        if (active && any_cross) load_cells<CPT>(out, gx);  // before the prefetch: it is awaited first
-        fetch_into(s + 2 * NSLOT, qx, qd);
-        if (active) {
-            const float *xw = stages + st * STAGE, *dw = xw + TL::WIN;
-            float dc[CPT], g[CPT];
+    using Buf = typename FetchLines<TL, TPS>::Buf;
+    // element e of round r of this slot; past the end of the chunk it is not `real`
+    auto sample = [&](int r, int e) { return s0 + (r * E + e) * NSLOT + slot; };
+    Buf px[E], pd[E];
+    // Loads and commits are unconditional (past the end of the chunk they repeat its last
+    // element, which nobody then uses): with branches around them the compiler cannot count the
+    // loads in flight and waits for ALL of them wherever it needs one.
+    auto fetch_round = [&](int r) {
 #pragma unroll
-            for (int c = 0; c < CPT; ++c) {
-                dc[c] = dw[pl.own + c];
-                g[c] = 0.f;
+        for (int e = 0; e < E; ++e) {
+            const long at = (long)min(sample(r, e), s1 - 1) * cells;
+            fx.fetch(x + at, px[e]);
+            fx.fetch(dsum + at, pd[e]);
+        }
+    };
+    auto commit_round = [&](int st) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            fx.template commit<1>(stages + st * STAGE + e * PAIR, px[e]);
+            fx.template commit<1>(stages + st * STAGE + e * PAIR + TL::WIN, pd[e]);
+        }
+    };
+    float gx[E][BS];  // row threads: dx of their row so far (the own block's part)
+    int r_prev = -1;
+    // the round before: its parts are all in slab `st` by now (a barrier lies in between)
+    auto finish_prev = [&](int st) {
+        if (r_prev >= 0 && is_row) {
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                const int s = sample(r_prev, e);
+                const float *slab = slabs + (st * E + e) * TPS;
+                // fixed order per cell: k faces, then i face, then j face
+                gx[e][0] += slab[4 * FS + ri * BS + rj];
+                gx[e][BS - 1] += slab[5 * FS + ri * BS + rj];
+                if (ri_edge) {
+                    float part[BS];
+                    load_cells<BS>(slab + (ri == 0 ? 0 : 1) * FS + rj * BS, part);
+#pragma unroll
+                    for (int c = 0; c < BS; ++c) gx[e][c] += part[c];
+                }
+                if (rj_edge) {
+                    float part[BS];
+                    load_cells<BS>(slab + (rj == 0 ? 2 : 3) * FS + ri * BS, part);
+#pragma unroll
+                    for (int c = 0; c < BS; ++c) gx[e][c] += part[c];
+                }
+                if (s < s1) store_cells<BS>(dx + (long)s * cells + grow, gx[e]);
             }
-            for_each_row<TL, CPT, kCrossDepth>(dw + pl.row00, [&](int r, const float (&dv)[CPT + 2]) {
-#pragma unroll
-                for (int cc = 0; cc < 3; ++cc)
-#pragma unroll
-                    for (int c = 0; c < CPT; ++c) g[c] = fmaf(vx[r * 3 + cc][c], dv[c + cc], g[c]);
-            });
-            for_each_row<TL, CPT, kCrossDepth>(xw + pl.row00, [&](int r, const float (&xv)[CPT + 2]) {
-#pragma unroll
-                for (int cc = 0; cc < 3; ++cc)
-#pragma unroll
-                    for (int c = 0; c < CPT; ++c)
-                        cw[r * 3 + cc][c] = fmaf(dc[c], xv[c + cc], cw[r * 3 + cc][c]);
-            });
-            if (any_cross) {
-#pragma unroll
-                for (int c = 0; c < CPT; ++c) gx[c] += g[c];
-                store_cells<CPT>(out, gx);
-            }
         }
-        commit_from(s + NSLOT, st ^ 1, px, pd);
+        r_prev = -1;
     };
-    fetch_into(s0 + pl.slot, ax, ad);
-    fetch_into(s0 + pl.slot + NSLOT, bx, bd);
-    commit_from(s0 + pl.slot, 0, ax, ad);
-    for (int sb = s0; sb < s1; sb += 2 * NSLOT) {
-        element(sb + pl.slot, 0, bx, bd, ax, ad);
-        element(sb + pl.slot + NSLOT, 1, ax, ad, bx, bd);  // may lie past the end: idles
+    const int rounds = (s1 - s0 + E * NSLOT - 1) / (E * NSLOT);
+    fetch_round(0);
+    commit_round(0);
+    for (int r = 0; r < rounds; ++r) {
+        const int st = r & 1;
+        lds_barrier();  // stage `st` and slab `st ^ 1` are complete; their old readers are done
+        finish_prev(st ^ 1);
+        if (is_row) {  // requested before the prefetch, so that they are awaited first
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+                load_cells<BS>(dx + (long)min(sample(r, e), s1 - 1) * cells + grow, gx[e]);
+        }
+        fetch_round(r + 1);
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const float *xw = stages + st * STAGE + e * PAIR, *dw = xw + TL::WIN;
+            const float dc = dw[own];
+            float dh[9], xh[9];
+#pragma unroll
+            for (int pq = 0; pq < 9; ++pq) {
+                dh[pq] = dw[hoff[pq]];
+                xh[pq] = xw[hoff[pq]];
+            }
+            const bool real = sample(r, e) < s1;
+            float g = 0.f;
+#pragma unroll
+            for (int pq = 0; pq < 9; ++pq) {
+                g = fmaf(vx[pq], dh[pq], g);
+                cw[pq] = fmaf(real ? dc : 0.f, xh[pq], cw[pq]);
+            }
+            slabs[(st * E + e) * TPS + lane] = g;
+        }
+        r_prev = r;
+        commit_round(st ^ 1);
     }
+    lds_barrier();
+    finish_prev((rounds - 1) & 1);
 
     if (NSLOT > 1) {
         float *red = lds;  // NSLOT * TPS floats, reused value by value
 #pragma unroll
-        for (int t = 0; t < 27; ++t)
+        for (int pq = 0; pq < 9; ++pq) {
+            lds_barrier();
+            red[slot * TPS + lane] = cw[pq];
+            lds_barrier();
+            if (slot == 0) {
 #pragma unroll
-            for (int c = 0; c < CPT; ++c) {
-                lds_barrier();
-                red[pl.slot * TL::TPS + pl.lane] = cw[t][c];
-                lds_barrier();
-                if (pl.slot == 0) {
-#pragma unroll
-                    for (int q = 1; q < NSLOT; ++q) cw[t][c] += red[q * TL::TPS + pl.lane];
-                }
+                for (int q = 1; q < NSLOT; ++q) cw[pq] += red[q * TPS + lane];
             }
-        if (pl.slot != 0) return;
+        }
+        if (slot != 0) return;
     }
-    // every tap that leaves the block is committed, also where it reads the zero padding outside
-    // the grid (its gradient is exactly zero and a store-mode caller expects every entry written)
-    commit_grads<27, CPT>(
-        dweight, cw, param_mode, [&](int t, int c) { return t * cells + pl.gc + c; },
-        leaves_block);
+    // every pair is committed, also where its tap reads the zero padding outside the grid (the
+    // gradient is exactly zero and a store-mode caller expects every entry written)
+#pragma unroll
+    for (int pq = 0; pq < 9; ++pq) {
+        const int dp = pq / 3 - 1, dq = pq % 3 - 1;
+        const int di = axis == 0 ? out : dp;
+        const int dj = axis == 0 ? dp : axis == 1 ? out : dq;
+        const int dk = axis == 2 ? out : dq;
+        const int t = (di + 1) * 9 + (dj + 1) * 3 + (dk + 1);
+        if (mine[pq]) {
+            if (param_mode != kParamAtomic) dweight[t * cells + gcell] = cw[pq];
+            else unsafeAtomicAdd(dweight + t * cells + gcell, cw[pq]);
+        }
+    }
 }
 
 __global__ void fill_zero_f32(float *p, long n) {
@@ -809,8 +921,8 @@ template <int BS, int CPT, int NSLOT, int ACT> int launch_fwd(const StepArgs &a,
 constexpr size_t kMaxLds = 160 * 1024;
 
 // the cross-block kernel's own shapes (it shares the main kernel's blocks and batch chunks)
-constexpr int kCrossCpt8 = 2, kCrossSlots8 = 1;  // bs=8: 256 threads
-constexpr int kCrossCpt4 = 1, kCrossSlots4 = 4;  // bs=4: four one-wave slots
+constexpr int kCrossSlots8 = 1, kCrossElems8 = 2;  // bs=8: 384 threads, one wave per face
+constexpr int kCrossSlots4 = 4, kCrossElems4 = 2;  // bs=4: four slots of 96 threads
 
 template <int BS, int CPT, int NSLOT, int ACT> int launch_bwd(const StepArgs &a, hipStream_t st) {
     using TL = Tile<BS, CPT>;
@@ -858,9 +970,10 @@ template <int BS, int CPT, int NSLOT, int ACT> int launch_bwd(const StepArgs &a,
     if (int rc = check_launch("step_bwd_fast")) return rc;
     // same blocks, same batch chunks, same way of committing parameter gradients (the two
     // kernels write disjoint entries of dweight)
-    constexpr int XCPT = BS == 8 ? kCrossCpt8 : kCrossCpt4, XSLOT = BS == 8 ? kCrossSlots8 : kCrossSlots4;
-    hipLaunchKernelGGL((step_bwd_cross<BS, XCPT, XSLOT>), dim3(padded_grid(p.nblk, p.nchunk)),
-                       dim3(Tile<BS, XCPT>::TPS * XSLOT), 0, st, (const float *)a.weight,
+    constexpr int XSLOT = BS == 8 ? kCrossSlots8 : kCrossSlots4;
+    constexpr int XE = BS == 8 ? kCrossElems8 : kCrossElems4;
+    hipLaunchKernelGGL((step_bwd_cross<BS, XSLOT, XE>), dim3(padded_grid(p.nblk, p.nchunk)),
+                       dim3(6 * BS * BS * XSLOT), 0, st, (const float *)a.weight,
                        (const float *)a.x, (const float *)a.workspace, (float *)a.dweight,
                        (float *)a.dx, a.B, a.M, a.N, a.K, p.nblk, p.nchunk, p.chunk_len, param_mode);
     if (int rc = check_launch("step_bwd_cross")) return rc;
