@@ -20,7 +20,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor peak
 
 
-def gpu_run(wl, steps, warmup):
+def gpu_run(wl, steps, warmup, fused):
     import torch
 
     from gridnet_amd.configs import make_inputs
@@ -30,7 +30,8 @@ def gpu_run(wl, steps, warmup):
     torch.cuda.set_device(dev)
     t = {k: v.to(dev) for k, v in make_inputs(wl, seed=0).items()}
     run = BodyRunner(t["weight"], t["bias"], t["scale"], t["gamma"], t["beta"], wl.batch, wl.inner,
-                     wl.outer, wl.block_size, wl.activation, wl.normalize, backward=wl.backward)
+                     wl.outer, wl.block_size, wl.activation, wl.normalize, backward=wl.backward,
+                     fused=fused)
 
     def one_step():
         run.forward(t["x0"])
@@ -121,6 +122,10 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="C3")
+    ap.add_argument("--path", choices=("steps", "fused"), default="steps",
+                    help="steps: one call per step and per LayerNorm, as the reference's callers do "
+                         "(the faster of the two on MI355X as measured); fused: the entry points "
+                         "with the LayerNorm folded into the step kernels")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -129,8 +134,12 @@ def main():
     from gridnet_amd.configs import WORKLOADS
 
     wl = WORKLOADS[args.workload]
-    wall, kernel_s = gpu_run(wl, args.steps, args.warmup)
+    fused = args.path == "fused" and not wl.normalize and wl.inner >= 1
+    wall, kernel_s = gpu_run(wl, args.steps, args.warmup, fused)
     bytes_ = wl.algorithmic_bytes()
+    if fused:  # a fused entry point does the work of the step AND of the LayerNorm beside it
+        bytes_["step_fwd"] += bytes_["ln_fwd"]
+        bytes_["step_bwd"] += bytes_["ln_bwd"]
     dominant = max(kernel_s, key=lambda k: kernel_s[k])
     # HBM bytes per call of that entry point, from the committed rocprofv3 --pmc summary
     # (FETCH_SIZE and WRITE_SIZE runs, scaled by a copy kernel of known size); null if absent
@@ -156,7 +165,8 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {"workload": wl.name, "activation": wl.activation, "normalize": wl.normalize,
-                   "pass": "fwd+bwd" if wl.backward else "fwd"},
+                   "pass": "fwd+bwd" if wl.backward else "fwd",
+                   "path": "fused step+LayerNorm entry points" if fused else "step and LayerNorm calls"},
         "hbm_roofline_frac_whole_step": bytes_["total"] / wall / (HBM_PEAK_GBS * 1e9),
         "entry_point_ms": {k: v * 1e3 for k, v in kernel_s.items()},
         "roofline": {

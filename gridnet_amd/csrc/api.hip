@@ -200,4 +200,140 @@ int gridnet_hip_layernorm_backward(int dtype, const void *dy, const void *x, con
     return layernorm_backward(a, (hipStream_t)stream);
 }
 
+// ---- network body with the LayerNorm folded into the step kernels -------------------------
+static int check_fused(const StepArgs &a, bool backward) {
+    if (a.dtype != GRIDNET_F32)
+        return fail(GRIDNET_ERR_ARGUMENT, "the fused body is float32 only (dtype id %d)", a.dtype);
+    if (int rc = check_step(a, backward)) return rc;
+    if (a.inner < 1)
+        return fail(GRIDNET_ERR_ARGUMENT, "the fused body needs at least one inner iteration");
+    if (!step_fast_supports(a, backward))
+        return fail(GRIDNET_ERR_ARGUMENT,
+                    "the fused body does not cover this problem (inner=%d block_size=%d): use the "
+                    "step and LayerNorm entry points",
+                    a.inner, a.block_size);
+    return GRIDNET_OK;
+}
+
+static size_t fused_forward_workspace(const StepArgs &a) {
+    const size_t nblk = (size_t)(a.M / a.block_size) * (a.N / a.block_size) * (a.K / a.block_size);
+    return (size_t)a.B * nblk * step_fast_forward_parts(a.block_size) * 2 * sizeof(float);
+}
+
+// backward workspace: [D of every cell | partial sums of the cross-block kernel]
+static size_t fused_backward_dsum(const StepArgs &a) {
+    return (step_fast_backward_workspace(a) + 255) / 256 * 256;
+}
+static size_t fused_backward_parts(const StepArgs &a) {
+    const size_t nblk = (size_t)(a.M / a.block_size) * (a.N / a.block_size) * (a.K / a.block_size);
+    return (size_t)a.B * nblk * step_fast_backward_parts(a.block_size) * 2 * sizeof(float);
+}
+
+size_t gridnet_hip_fused_workspace_bytes(int B, int M, int N, int K, int inner, int block_size,
+                                         int backward) {
+    StepArgs a{};
+    a.dtype = GRIDNET_F32; a.B = B; a.M = M; a.N = N; a.K = K; a.inner = inner;
+    a.block_size = block_size; a.activation = GRIDNET_ACT_RELU;
+    if (B <= 0 || M <= 0 || N <= 0 || K <= 0 || (block_size != 4 && block_size != 8)) return 0;
+    if (!backward) return fused_forward_workspace(a);
+    return fused_backward_dsum(a) + fused_backward_parts(a);
+}
+
+int gridnet_hip_fused_forward(int dtype, const void *weight, const void *bias, const void *scale,
+                              const void *gamma, const void *beta, const void *x,
+                              const void *x_stats, void *y_raw, void *y_stats, int B, int M, int N,
+                              int K, int inner, int block_size, double ln_eps, int activation,
+                              void *workspace, size_t workspace_bytes, void *stream) {
+    StepArgs a{};
+    a.dtype = dtype; a.weight = weight; a.bias = bias; a.scale = scale; a.x = x; a.y = y_raw;
+    a.B = B; a.M = M; a.N = N; a.K = K; a.inner = inner; a.block_size = block_size;
+    a.activation = activation;
+    if (int rc = check_fused(a, false)) return rc;
+    if (B == 0) return GRIDNET_OK;
+    if (!gamma || !beta || !y_stats) return fail(GRIDNET_ERR_ARGUMENT, "null pointer");
+    const size_t need = fused_forward_workspace(a);
+    if (!workspace || workspace_bytes < need)
+        return fail(GRIDNET_ERR_WORKSPACE, "fused forward needs %zu bytes of workspace, got %zu", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    hipStream_t st = (hipStream_t)stream;
+    a.ln.gamma = (const float *)gamma;
+    a.ln.beta = (const float *)beta;
+    a.ln.x_stats = (const float *)x_stats;
+    a.ln.y_part = (float *)workspace;
+    if (int rc = step_forward_fast(a, st)) return rc;
+    const int nblk = (M / block_size) * (N / block_size) * (K / block_size);
+    return layernorm_finalize_stats((const float *)workspace, nblk * step_fast_forward_parts(block_size),
+                                    step_fast_forward_part_count(block_size), (float *)y_stats, B,
+                                    ln_eps, st);
+}
+
+int gridnet_hip_layernorm_apply(int dtype, const void *x, const void *stats, const void *gamma,
+                                const void *beta, void *y, int B, long n, void *stream) {
+    if (dtype != GRIDNET_F32)
+        return fail(GRIDNET_ERR_ARGUMENT, "layernorm_apply is float32 only (dtype id %d)", dtype);
+    if (B < 0 || n <= 0) return fail(GRIDNET_ERR_ARGUMENT, "bad shape B=%d n=%ld", B, n);
+    if (B == 0) return GRIDNET_OK;
+    if (!x || !stats || !gamma || !beta || !y) return fail(GRIDNET_ERR_ARGUMENT, "null pointer");
+    return layernorm_apply_stats((const float *)x, (const float *)stats, (const float *)gamma,
+                                 (const float *)beta, (float *)y, B, n, (hipStream_t)stream);
+}
+
+int gridnet_hip_layernorm_backward_sums(int dtype, const void *dy, const void *x, const void *stats,
+                                        const void *gamma, void *sums, int B, long n,
+                                        void *workspace, size_t workspace_bytes, void *stream) {
+    if (dtype != GRIDNET_F32)
+        return fail(GRIDNET_ERR_ARGUMENT, "layernorm_backward_sums is float32 only (dtype id %d)", dtype);
+    if (B < 0 || n <= 0) return fail(GRIDNET_ERR_ARGUMENT, "bad shape B=%d n=%ld", B, n);
+    if (B == 0) return GRIDNET_OK;
+    if (!dy || !x || !stats || !gamma || !sums) return fail(GRIDNET_ERR_ARGUMENT, "null pointer");
+    const size_t need = layernorm_workspace(GRIDNET_F32, B, n);
+    if (!workspace || workspace_bytes < need)
+        return fail(GRIDNET_ERR_WORKSPACE, "layernorm needs %zu bytes of workspace, got %zu", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    return layernorm_backward_sums((const float *)dy, (const float *)x, (const float *)stats,
+                                   (const float *)gamma, (float *)sums, B, n, (float *)workspace,
+                                   (hipStream_t)stream);
+}
+
+int gridnet_hip_fused_backward(int dtype, const void *weight, const void *bias, const void *scale,
+                               const void *gamma, const void *beta, const void *x,
+                               const void *x_stats, const void *dy, const void *y_raw,
+                               const void *y_stats, const void *y_sums, void *dweight, void *dbias,
+                               void *dscale, void *dgamma, void *dbeta, void *dx, void *x_sums, int B,
+                               int M, int N, int K, int inner, int block_size, int activation,
+                               int flags, void *workspace, size_t workspace_bytes, void *stream) {
+    StepArgs a{};
+    a.dtype = dtype; a.weight = weight; a.bias = bias; a.scale = scale; a.x = x; a.dy = dy;
+    a.dweight = dweight; a.dbias = dbias; a.dscale = dscale; a.dx = dx;
+    a.B = B; a.M = M; a.N = N; a.K = K; a.inner = inner; a.block_size = block_size;
+    a.activation = activation;
+    a.flags = (flags & GRIDNET_OVERWRITE_PARAMS) | GRIDNET_OVERWRITE_DX;  // dx is always written
+    a.ln.gamma = (const float *)gamma;  // before the checks: the LDS budget depends on it
+    if (int rc = check_fused(a, true)) return rc;
+    if (B == 0) return GRIDNET_OK;
+    if (!gamma || !beta || !y_raw || !y_stats || !y_sums || !dgamma || !dbeta)
+        return fail(GRIDNET_ERR_ARGUMENT, "null pointer");
+    if ((x_stats == nullptr) != (x_sums == nullptr))
+        return fail(GRIDNET_ERR_ARGUMENT, "x_stats and x_sums go together: both or neither");
+    const size_t dsum_bytes = fused_backward_dsum(a), need = dsum_bytes + fused_backward_parts(a);
+    if (!workspace || workspace_bytes < need)
+        return fail(GRIDNET_ERR_WORKSPACE, "fused backward needs %zu bytes of workspace, got %zu", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    hipStream_t st = (hipStream_t)stream;
+    a.workspace = workspace; a.workspace_bytes = dsum_bytes;
+    a.ln.beta = (const float *)beta;
+    a.ln.x_stats = (const float *)x_stats;
+    a.ln.y_raw = (const float *)y_raw;
+    a.ln.y_stats = (const float *)y_stats;
+    a.ln.y_sums = (const float *)y_sums;
+    a.ln.dgamma = (float *)dgamma;
+    a.ln.dbeta = (float *)dbeta;
+    a.ln.x_part = x_stats ? (float *)((char *)workspace + dsum_bytes) : nullptr;
+    if (int rc = step_backward_fast(a, st)) return rc;
+    if (!x_stats) return GRIDNET_OK;
+    const int nblk = (M / block_size) * (N / block_size) * (K / block_size);
+    return layernorm_finalize_sums(a.ln.x_part, nblk * step_fast_backward_parts(block_size),
+                                   (long)M * N * K, (float *)x_sums, B, st);
+}
+
 }  // extern "C"

@@ -7,6 +7,25 @@
 
 namespace gridnet {
 
+// LayerNorm folded into the step kernels: one outer step of the body "update step, then
+// per-sample LayerNorm over the grid" without a pass of its own for the LayerNorm.  A step reads
+// the RAW output of the step before it (before that step's LayerNorm) and normalises it while
+// loading; it writes its own raw output and what the next step needs to do the same.  All
+// members may be null; statistics are (mean, rstd) pairs, sums are the two per-sample means of
+// the LayerNorm backward, one pair per batch element, fp32.
+struct LnFold {
+    const float *gamma, *beta;  // [M,N,K]
+    const float *x_stats;       // [B,2]: LayerNorm applied to x on load; null: x is used as is
+    float *y_part;              // forward: partial (mean, M2) of the output, one pair per 16-lane
+                                // group, [B, nblk, groups, 2]
+    // backward: the incoming gradient is with respect to LayerNorm(y_raw)
+    const float *y_raw;         // [B,M,N,K] this step's forward output before its LayerNorm
+    const float *y_stats;       // [B,2]
+    const float *y_sums;        // [B,2]: mean(g), mean(g * yhat) with g = gamma * incoming gradient
+    float *dgamma, *dbeta;      // [M,N,K], summed over the batch, committed like dbias
+    float *x_part;              // partial sums for the LayerNorm backward of x: [B, nblk, parts, 2]
+};
+
 struct StepArgs {
     int dtype;
     const void *weight, *bias, *scale, *x;
@@ -18,6 +37,7 @@ struct StepArgs {
     int normalize, activation, flags;
     void *workspace;
     size_t workspace_bytes;
+    LnFold ln;  // all null: the plain step
 };
 
 // How a workgroup commits its parameter gradients.
@@ -48,12 +68,29 @@ bool step_fast_supports(const StepArgs &a, bool backward);
 size_t step_fast_backward_workspace(const StepArgs &a);
 int step_forward_fast(const StepArgs &a, hipStream_t st);
 int step_backward_fast(const StepArgs &a, hipStream_t st);
+// partial statistics per (block, batch element) that the kernels above write when asked to
+int step_fast_forward_parts(int block_size);   // (mean, M2) pairs, each over forward_part_count cells
+int step_fast_forward_part_count(int block_size);
+int step_fast_backward_parts(int block_size);  // (sum g, sum g*xhat) pairs
 
 // gated_generic.hip (weight [27,2,M,N,K], bias [2,M,N,K]; scale, eps, normalize unused)
 int gated_forward(const StepArgs &a, hipStream_t st);
 int gated_backward(const StepArgs &a, hipStream_t st);
 
 // layernorm.hip
+// (mean, M2) pairs over `count` cells each -> (mean, rstd) per sample
+int layernorm_finalize_stats(const float *part, int parts_per_sample, int count, float *stats, int B,
+                             double eps, hipStream_t st);
+// (sum, sum) pairs -> their means over n cells per sample
+int layernorm_finalize_sums(const float *part, int parts_per_sample, long n, float *sums, int B,
+                            hipStream_t st);
+// y = (x - mean) * rstd * gamma + beta with given statistics
+int layernorm_apply_stats(const float *x, const float *stats, const float *gamma, const float *beta,
+                          float *y, int B, long n, hipStream_t st);
+// the two per-sample means of the LayerNorm backward from interleaved (mean, rstd) statistics;
+// `partial` holds layernorm_workspace() bytes
+int layernorm_backward_sums(const float *dy, const float *x, const float *stats, const float *gamma,
+                            float *sums, int B, long n, float *partial, hipStream_t st);
 size_t layernorm_workspace(int dtype, int B, long n);
 int layernorm_forward(const LayerNormArgs &a, hipStream_t st);
 int layernorm_backward(const LayerNormArgs &a, hipStream_t st);

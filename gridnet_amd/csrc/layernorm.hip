@@ -152,11 +152,11 @@ __global__ __launch_bounds__(kLnThreads) void ln_bwd_partial(const T *__restrict
                                                              const T *__restrict__ mean,
                                                              const T *__restrict__ rstd,
                                                              T *__restrict__ partial, long n,
-                                                             int nchunk) {
+                                                             int nchunk, int stat_stride) {
     __shared__ T red[kLnThreads / kWave];
     const int tid = threadIdx.x, chunk = blockIdx.x, b = blockIdx.y;
     const long start = (long)chunk * kLnChunk;
-    const T mu = mean[b], rs = rstd[b];
+    const T mu = mean[b * stat_stride], rs = rstd[b * stat_stride];
     T g[kLnPerThread], xv[kLnPerThread], gm[kLnPerThread];
     load_chunk<T, VEC>(dy + (long)b * n, start, n, tid, g);
     load_chunk<T, VEC>(x + (long)b * n, start, n, tid, xv);
@@ -239,6 +239,98 @@ __global__ __launch_bounds__(kLnThreads) void ln_bwd_apply(
     }
 }
 
+// ---- pieces of the LayerNorm folded into the step kernels (fp32) ---------------------------
+// The step kernels leave per-group partial results; these small kernels turn them into the
+// per-sample numbers, in double and in a fixed order (one workgroup per sample).
+
+constexpr int kFinThreads = 1024;
+constexpr int kFinUnroll = 4;  // pairs a thread requests before it uses any
+
+// (mean_i, M2_i) over `count` cells each -> (mean, rstd): mean = avg(mean_i),
+// M2 = sum(M2_i + count (mean_i - mean)^2)  (exact pairwise-combination formula).
+__global__ __launch_bounds__(kFinThreads) void ln_finalize_stats(const float *__restrict__ part,
+                                                                 int parts, int count,
+                                                                 float *__restrict__ stats, double eps) {
+    __shared__ double red[kFinThreads / kWave];
+    const int tid = threadIdx.x, b = blockIdx.x;
+    const float2 *ps = reinterpret_cast<const float2 *>(part) + (long)b * parts;
+    double s = 0.0, q = 0.0, qm = 0.0;
+    // one pass: sum(mean_i), sum(M2_i), sum(mean_i^2); means are O(1) and few thousand, so the
+    // squares lose nothing in double
+    for (int i0 = tid; i0 < parts; i0 += kFinThreads * kFinUnroll) {
+        float2 v[kFinUnroll];
+#pragma unroll
+        for (int k = 0; k < kFinUnroll; ++k) {
+            const int i = i0 + k * kFinThreads;
+            v[k] = i < parts ? ps[i] : make_float2(0.f, 0.f);
+        }
+#pragma unroll
+        for (int k = 0; k < kFinUnroll; ++k) {
+            s += (double)v[k].x;
+            q += (double)v[k].y;
+            qm += (double)v[k].x * (double)v[k].x;
+        }
+    }
+    s = block_sum(s, red, tid, kFinThreads);
+    q = block_sum(q, red, tid, kFinThreads);
+    qm = block_sum(qm, red, tid, kFinThreads);
+    if (tid == 0) {
+        const double mean = s / parts;
+        // sum count (mean_i - mean)^2 = count (sum mean_i^2 - parts mean^2)
+        const double var = (q + count * (qm - parts * mean * mean)) / ((double)parts * count);
+        stats[2 * b] = (float)mean;
+        stats[2 * b + 1] = (float)(1.0 / sqrt((var > 0.0 ? var : 0.0) + eps));
+    }
+}
+
+// (s1_i, s2_i) -> (sum s1 / n, sum s2 / n)
+__global__ __launch_bounds__(kFinThreads) void ln_finalize_sums(const float *__restrict__ part,
+                                                                int parts, long n,
+                                                                float *__restrict__ sums) {
+    __shared__ double red[kFinThreads / kWave];
+    const int tid = threadIdx.x, b = blockIdx.x;
+    const float2 *ps = reinterpret_cast<const float2 *>(part) + (long)b * parts;
+    double s1 = 0.0, s2 = 0.0;
+    for (int i0 = tid; i0 < parts; i0 += kFinThreads * kFinUnroll) {
+        float2 v[kFinUnroll];
+#pragma unroll
+        for (int k = 0; k < kFinUnroll; ++k) {
+            const int i = i0 + k * kFinThreads;
+            v[k] = i < parts ? ps[i] : make_float2(0.f, 0.f);
+        }
+#pragma unroll
+        for (int k = 0; k < kFinUnroll; ++k) {
+            s1 += (double)v[k].x;
+            s2 += (double)v[k].y;
+        }
+    }
+    s1 = block_sum(s1, red, tid, kFinThreads);
+    s2 = block_sum(s2, red, tid, kFinThreads);
+    if (tid == 0) {
+        sums[2 * b] = (float)(s1 / (double)n);
+        sums[2 * b + 1] = (float)(s2 / (double)n);
+    }
+}
+
+// y = (x - mean) * rstd * gamma + beta with statistics that are already known
+template <bool VEC>
+__global__ __launch_bounds__(kLnThreads) void ln_apply_stats(const float *__restrict__ x,
+                                                             const float *__restrict__ stats,
+                                                             const float *__restrict__ gamma,
+                                                             const float *__restrict__ beta,
+                                                             float *__restrict__ y, long n) {
+    const int tid = threadIdx.x, chunk = blockIdx.x, b = blockIdx.y;
+    const float mean = stats[2 * b], rstd = stats[2 * b + 1];
+    const long start = (long)chunk * kLnChunk;
+    float r[kLnPerThread], gm[kLnPerThread], bt[kLnPerThread];
+    load_chunk<float, VEC>(x + (long)b * n, start, n, tid, r);
+    load_chunk<float, VEC>(gamma, start, n, tid, gm);
+    load_chunk<float, VEC>(beta, start, n, tid, bt);
+#pragma unroll
+    for (int i = 0; i < kLnPerThread; ++i) r[i] = (r[i] - mean) * rstd * gm[i] + bt[i];
+    store_chunk<float, VEC>(y + (long)b * n, start, n, tid, r);
+}
+
 inline int chunks_of(long n) { return (int)((n + kLnChunk - 1) / kLnChunk); }
 
 template <typename T> bool aligned4(const void *p) { return ((uintptr_t)p % (4 * sizeof(T))) == 0; }
@@ -276,11 +368,11 @@ template <typename T> int backward_t(const LayerNormArgs &a, hipStream_t st) {
     if (vec)
         hipLaunchKernelGGL((ln_bwd_partial<T, true>), grid, block, 0, st, (const T *)a.dy,
                            (const T *)a.x, (const T *)a.gamma, (const T *)a.mean_in,
-                           (const T *)a.rstd_in, partial, a.n, nchunk);
+                           (const T *)a.rstd_in, partial, a.n, nchunk, 1);
     else
         hipLaunchKernelGGL((ln_bwd_partial<T, false>), grid, block, 0, st, (const T *)a.dy,
                            (const T *)a.x, (const T *)a.gamma, (const T *)a.mean_in,
-                           (const T *)a.rstd_in, partial, a.n, nchunk);
+                           (const T *)a.rstd_in, partial, a.n, nchunk, 1);
     hipLaunchKernelGGL((ln_bwd_finalize<T>), dim3(a.B), block, 0, st, partial, sample_means, a.n,
                        nchunk);
 #define GRIDNET_LN_APPLY(V, ACC)                                                                   \
@@ -299,6 +391,46 @@ template <typename T> int backward_t(const LayerNormArgs &a, hipStream_t st) {
 }
 
 }  // namespace
+
+int layernorm_finalize_stats(const float *part, int parts_per_sample, int count, float *stats, int B,
+                             double eps, hipStream_t st) {
+    hipLaunchKernelGGL(ln_finalize_stats, dim3(B), dim3(kFinThreads), 0, st, part, parts_per_sample,
+                       count, stats, eps);
+    return check_launch("ln_finalize_stats");
+}
+
+int layernorm_finalize_sums(const float *part, int parts_per_sample, long n, float *sums, int B,
+                            hipStream_t st) {
+    hipLaunchKernelGGL(ln_finalize_sums, dim3(B), dim3(kFinThreads), 0, st, part, parts_per_sample, n,
+                       sums);
+    return check_launch("ln_finalize_sums");
+}
+
+int layernorm_apply_stats(const float *x, const float *stats, const float *gamma, const float *beta,
+                          float *y, int B, long n, hipStream_t st) {
+    const bool vec = n % 4 == 0 && aligned4<float>(x) && aligned4<float>(y) &&
+                     aligned4<float>(gamma) && aligned4<float>(beta);
+    dim3 grid(chunks_of(n), B), block(kLnThreads);
+    if (vec) hipLaunchKernelGGL((ln_apply_stats<true>), grid, block, 0, st, x, stats, gamma, beta, y, n);
+    else hipLaunchKernelGGL((ln_apply_stats<false>), grid, block, 0, st, x, stats, gamma, beta, y, n);
+    return check_launch("ln_apply_stats");
+}
+
+int layernorm_backward_sums(const float *dy, const float *x, const float *stats, const float *gamma,
+                            float *sums, int B, long n, float *partial, hipStream_t st) {
+    const int nchunk = chunks_of(n);
+    const bool vec = n % 4 == 0 && aligned4<float>(x) && aligned4<float>(dy) && aligned4<float>(gamma);
+    dim3 grid(nchunk, B), block(kLnThreads);
+    if (vec)
+        hipLaunchKernelGGL((ln_bwd_partial<float, true>), grid, block, 0, st, dy, x, gamma, stats,
+                           stats + 1, partial, n, nchunk, 2);
+    else
+        hipLaunchKernelGGL((ln_bwd_partial<float, false>), grid, block, 0, st, dy, x, gamma, stats,
+                           stats + 1, partial, n, nchunk, 2);
+    hipLaunchKernelGGL((ln_bwd_finalize<float>), dim3(B), block, 0, st, (const float *)partial, sums, n,
+                       nchunk);
+    return check_launch("layernorm_backward_sums");
+}
 
 size_t layernorm_workspace(int dtype, int B, long n) {
     const size_t elt = dtype == GRIDNET_F64 ? 8 : 4;

@@ -63,6 +63,29 @@ __device__ __forceinline__ void lds_barrier() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// Sum over the 16 lanes of a DPP row (lanes 16q .. 16q+15), delivered to every one of them:
+// four rotate-and-add steps on the vector ALU, no LDS traffic.
+__device__ __forceinline__ float row16_sum(float v) {
+#define GRIDNET_ROR(n) \
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x120 + (n), 0xf, 0xf, false))
+    GRIDNET_ROR(8);
+    GRIDNET_ROR(4);
+    GRIDNET_ROR(2);
+    GRIDNET_ROR(1);
+#undef GRIDNET_ROR
+    return v;
+}
+
+// Load p[i], i the same for the whole wave, as a VECTOR memory load.  Left alone the compiler
+// makes it a scalar load; those return out of order and share their counter with LDS, so one
+// that is still on its way stalls the next LDS access for a whole trip to memory -- and the
+// per-sample numbers loaded this way are requested an element ahead, in the middle of LDS work.
+__device__ __forceinline__ float load_ahead(const float *p, int i) {
+    int zero;
+    asm volatile("v_mov_b32 %0, 0" : "=v"(zero));
+    return p[i + zero];
+}
+
 // Wait for every global load issued so far (s_waitcnt vmcnt(0) only).  Placed once after the
 // per-workgroup parameter loads: with those known complete, the waits the compiler inserts
 // inside the batch loop no longer cover the prefetch of the next batch element as well.
@@ -226,6 +249,32 @@ template <typename TL, int NT = TL::TPS> struct Fetch {  // NT: threads of a slo
                 }
             }
     }
+    // The same, with the LayerNorm of the producer applied on the way in: an entry becomes
+    // (v - mean) * rstd * gamma + beta, gamma and beta read from windows `gwin`, `bwin` laid out
+    // like `win`; entries outside the grid stay zero.
+    template <int COPIES = 2>
+    __device__ __forceinline__ void commit_ln(float *win, const Buf &v, const float *gwin,
+                                              const float *bwin, float mean, float rstd) const {
+#pragma unroll
+        for (int e = 0; e < RPT; ++e)
+            if (loff[e] >= 0) {
+                const int at_end = loff[e] + (hi[e] ? HC : 0), at_cells = loff[e] + (hi[e] ? 0 : 1);
+                const float end = (ok[e] && edge_ok[e])
+                                      ? fmaf((v[e][HC] - mean) * rstd, gwin[at_end], bwin[at_end])
+                                      : 0.f;
+                float val[HC];
+#pragma unroll
+                for (int q = 0; q < HC; ++q)
+                    val[q] = ok[e] ? fmaf((v[e][q] - mean) * rstd, gwin[at_cells + q], bwin[at_cells + q])
+                                   : 0.f;
+#pragma unroll
+                for (int copy = 0; copy < COPIES; ++copy) {
+                    win[copy * TL::WIN + at_end] = end;
+#pragma unroll
+                    for (int q = 0; q < HC; ++q) win[copy * TL::WIN + at_cells + q] = val[q];
+                }
+            }
+    }
 };
 
 // The same job for a kernel whose time goes into the memory pipeline rather than arithmetic
@@ -265,7 +314,10 @@ template <typename TL, int NT> struct FetchLines {
 #pragma unroll
         for (int e = 0; e < RPT; ++e) load_cells<4>(xs + goff[e], v[e]);
     }
-    template <int COPIES = 2> __device__ __forceinline__ void commit(float *win, const Buf &v) const {
+    // entries are committed as (v - mean) * rstd (mean 0, rstd 1: as they are); zero outside the grid
+    template <int COPIES = 2>
+    __device__ __forceinline__ void commit(float *win, const Buf &v, float mean = 0.f,
+                                           float rstd = 1.f) const {
 #pragma unroll
         for (int e = 0; e < RPT; ++e) {
             const int kind = (meta[e] >> 12) & 3;
@@ -275,9 +327,10 @@ template <typename TL, int NT> struct FetchLines {
 #pragma unroll
                 for (int copy = 0; copy < COPIES; ++copy)
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) to[copy * TL::WIN + q] = ok ? v[e][q] : 0.f;
+                    for (int q = 0; q < 4; ++q)
+                        to[copy * TL::WIN + q] = ok ? (v[e][q] - mean) * rstd : 0.f;
             } else if (kind != 3) {
-                const float end = ok ? (kind == 1 ? v[e][3] : v[e][0]) : 0.f;
+                const float end = ok ? ((kind == 1 ? v[e][3] : v[e][0]) - mean) * rstd : 0.f;
 #pragma unroll
                 for (int copy = 0; copy < COPIES; ++copy) to[copy * TL::WIN] = end;
             }
@@ -338,31 +391,54 @@ __device__ __forceinline__ void stencil(const float *win, int row00, const float
 
 constexpr int kFwdDepth = 9;  // neighbour rows requested ahead of the arithmetic
 
-template <int BS, int CPT, int NSLOT, int ACT>
-__global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_fwd_fast(
+// LN: the variant with the LayerNorm of the network body folded in (see LnFold); without it
+// `ln` is ignored and the code is the plain step's.
+template <int BS, int CPT, int NSLOT, int ACT, bool LN>
+__global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) __attribute__((amdgpu_waves_per_eu(3)))
+void step_fwd_fast(
     const float *__restrict__ weight, const float *__restrict__ bias,
     const float *__restrict__ scale, const float *__restrict__ x, float *__restrict__ y, int B, int M,
-    int N, int K, int inner, int nblk, int nchunk, int chunk_len) {
+    int N, int K, int inner, int nblk, int nchunk, int chunk_len, LnFold ln) {
     using TL = Tile<BS, CPT>;
-    __shared__ __attribute__((aligned(16))) float lds[NSLOT * 2 * TL::WIN];
+    // per slot two copies of the window; then, for the folded LayerNorm, gamma and beta windows
+    __shared__ __attribute__((aligned(16))) float lds[NSLOT * 2 * TL::WIN + (LN ? 2 * TL::WIN : 0)];
 
     int blk, chunk;
     if (!split_block_id(blockIdx.x, nblk, nchunk, blk, chunk)) return;  // grid padding
     const Place<TL, CPT, NSLOT> pl(threadIdx.x, blk, N, K);
     const Fetch<TL> fx(pl.lane, pl.p0, pl.q0, pl.r0, M, N, K);
     float *win = lds + pl.slot * (2 * TL::WIN);
+    float *gwin = lds + NSLOT * 2 * TL::WIN, *bwin = gwin + TL::WIN;
     const long cells = (long)M * N * K;
+    const bool ln_in = LN && ln.x_stats != nullptr;  // x is the raw output of the step before
 
     float w[27][CPT], bv[CPT], rv[CPT];
 #pragma unroll
     for (int t = 0; t < 27; ++t) load_cells<CPT>(weight + t * cells + pl.gc, w[t]);
     load_cells<CPT>(bias + pl.gc, bv);
     load_cells<CPT>(scale + pl.gc, rv);
+    typename Fetch<TL>::Buf pre;
+    if (ln_in) {  // gamma and beta of the window, once per workgroup
+        if (pl.slot == 0) {
+            fx.fetch(ln.gamma, pre);
+            fx.template commit<1>(gwin, pre);
+            fx.fetch(ln.beta, pre);
+            fx.template commit<1>(bwin, pre);
+        }
+        lds_barrier();
+    }
     wait_global_loads();
 
     const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
-    typename Fetch<TL>::Buf pre;
-    if (s0 + pl.slot < s1) fx.fetch(x + (s0 + pl.slot) * cells, pre);
+    float pre_mean = 0.f, pre_rstd = 1.f;  // LayerNorm statistics of the element in `pre`
+    auto fetch_element = [&](int s) {
+        fx.fetch(x + s * cells, pre);
+        if (ln_in) {
+            pre_mean = load_ahead(ln.x_stats, 2 * s);
+            pre_rstd = load_ahead(ln.x_stats, 2 * s + 1);
+        }
+    };
+    if (s0 + pl.slot < s1) fetch_element(s0 + pl.slot);
     // The result of an element is stored one element late, after the next window has been
     // committed: the wait for the prefetched window would otherwise also wait for a store that
     // was issued an instant earlier (loads and stores share one in-order counter).
@@ -371,10 +447,13 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_fwd_fast(
     for (int sb = s0; sb < s1; sb += NSLOT) {
         const int s = sb + pl.slot;
         const bool active = s < s1;  // a slot past the end idles through the barriers
-        if (active) fx.commit(win, pre);
+        if (active) {
+            if (ln_in) fx.commit_ln(win, pre, gwin, bwin, pre_mean, pre_rstd);
+            else fx.commit(win, pre);
+        }
         lds_barrier();
         if (done_s >= 0) store_cells<CPT>(y + done_s * cells + pl.gc, done);
-        if (s + NSLOT < s1) fx.fetch(x + (s + NSLOT) * cells, pre);  // next element, in flight
+        if (s + NSLOT < s1) fetch_element(s + NSLOT);  // next element, in flight
         float cur[CPT];
         if (active) {
 #pragma unroll
@@ -391,6 +470,22 @@ __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) void step_fwd_fast(
                 }
             }
             lds_barrier();
+        }
+        if (LN && active && ln.y_part) {
+            // statistics of the result for the LayerNorm that follows: every group of 16 lanes
+            // leaves (mean, M2 about that mean) of its 16*CPT cells
+            float sum = 0.f, m2 = 0.f;
+#pragma unroll
+            for (int c = 0; c < CPT; ++c) sum += cur[c];
+            const float mean = row16_sum(sum) * (1.f / (16 * CPT));
+#pragma unroll
+            for (int c = 0; c < CPT; ++c) m2 = fmaf(cur[c] - mean, cur[c] - mean, m2);
+            m2 = row16_sum(m2);
+            if ((pl.lane & 15) == 0) {
+                float *to = ln.y_part + (((long)s * nblk + blk) * (TL::TPS / 16) + pl.lane / 16) * 2;
+                to[0] = mean;
+                to[1] = m2;
+            }
         }
         done_s = active ? s : -1;
 #pragma unroll
@@ -435,17 +530,22 @@ __device__ __forceinline__ void commit_grads(float *base, const float (&val)[R][
     }
 }
 
-template <int BS, int CPT, int NSLOT, int ACT>
+template <int BS, int CPT, int NSLOT, int ACT, bool LN>
 __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) __attribute__((amdgpu_waves_per_eu(2)))
 void step_bwd_fast(
     const float *__restrict__ weight, const float *__restrict__ bias,
     const float *__restrict__ scale, const float *__restrict__ x, const float *__restrict__ dy,
     float *__restrict__ dweight, float *__restrict__ dbias, float *__restrict__ dscale,
     float *__restrict__ dx, float *__restrict__ dsum_out, int B, int M, int N, int K, int inner,
-    int nblk, int nchunk, int chunk_len, int param_mode, int dx_accumulate) {
+    int nblk, int nchunk, int chunk_len, int param_mode, int dx_accumulate, LnFold ln) {
     using TL = Tile<BS, CPT>;
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int slot_floats = bwd_slot_floats<BS, CPT>(inner);
+    // LN (the LayerNorm of the network body folded in, see LnFold): `dy` is the gradient with
+    // respect to LayerNorm(y_raw) and is taken through that LayerNorm's backward as it is
+    // loaded (dgamma, dbeta fall out on the way); x is normalised as it is loaded when it is
+    // the raw output of the step before.
+    const bool ln_in = LN && ln.x_stats != nullptr;
 
     int blk, chunk;
     if (!split_block_id(blockIdx.x, nblk, nchunk, blk, chunk)) return;  // grid padding
@@ -454,6 +554,7 @@ void step_bwd_fast(
     float *win = lds + pl.slot * slot_floats;
     float *dwin = win + 2 * TL::WIN;
     float *hist = dwin + 2 * TL::WIN + pl.lane * CPT;  // + it*TPS*2*CPT (x_i), + TPS*CPT more (u_i)
+    float *gwin = lds + NSLOT * slot_floats, *bwin = gwin + TL::WIN;  // LN: gamma, beta windows
     const long cells = (long)M * N * K;
 
     // nw[t][c] belongs to the weight of the neighbour at c + off_t, where that lies in this block
@@ -484,6 +585,19 @@ void step_bwd_fast(
     load_cells<CPT>(scale + pl.gc, rv);
 #pragma unroll
     for (int c = 0; c < CPT; ++c) db[c] = dr[c] = 0.f;
+    float gam[CPT], dgam[CPT], dbet[CPT];
+    typename Fetch<TL>::Buf pre;
+    if (LN) {
+        load_cells<CPT>(ln.gamma + pl.gc, gam);
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) dgam[c] = dbet[c] = 0.f;
+        if (ln_in && pl.slot == 0) {  // gamma and beta of the window, once per workgroup
+            fx.fetch(ln.gamma, pre);
+            fx.template commit<1>(gwin, pre);
+            fx.fetch(ln.beta, pre);
+            fx.template commit<1>(bwin, pre);
+        }
+    }
 
     // delta windows: the halo stays zero for the whole kernel
     for (int idx = pl.lane; idx < 2 * TL::WIN; idx += TL::TPS) dwin[idx] = 0.f;
@@ -502,14 +616,52 @@ void step_bwd_fast(
             db[c] = dbias[pl.gc + c];
             dr[c] = dscale[pl.gc + c];
         }
+        if (LN) {
+            load_cells<CPT>(ln.dgamma + pl.gc, dgam);
+            load_cells<CPT>(ln.dbeta + pl.gc, dbet);
+        }
     }
 
     const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
-    typename Fetch<TL>::Buf pre;
-    float g[CPT];
+    // what is requested one element ahead: the x window, the incoming gradient of the owned
+    // cells and, for LN, the raw output there and the per-sample numbers of both LayerNorms
+    float g[CPT], gnext[CPT], ynext[CPT], nx_mean = 0.f, nx_rstd = 1.f, ny[4] = {0.f, 1.f, 0.f, 0.f};
+    auto fetch_element = [&](int s) {
+        fx.fetch(x + s * cells, pre);
+        load_cells<CPT>(dy + s * cells + pl.gc, gnext);
+        if (LN) {
+            load_cells<CPT>(ln.y_raw + s * cells + pl.gc, ynext);
+            ny[0] = load_ahead(ln.y_stats, 2 * s);
+            ny[1] = load_ahead(ln.y_stats, 2 * s + 1);
+            ny[2] = load_ahead(ln.y_sums, 2 * s);
+            ny[3] = load_ahead(ln.y_sums, 2 * s + 1);
+            if (ln_in) {
+                nx_mean = load_ahead(ln.x_stats, 2 * s);
+                nx_rstd = load_ahead(ln.x_stats, 2 * s + 1);
+            }
+        }
+    };
+    // the element just fetched becomes the current one: its gradient (through the LayerNorm
+    // backward for LN) and its window
+    auto take_element = [&]() {
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) {
+            if (LN) {
+                const float yh = (ynext[c] - ny[0]) * ny[1];
+                dgam[c] = fmaf(gnext[c], yh, dgam[c]);
+                dbet[c] += gnext[c];
+                g[c] = ny[1] * (gam[c] * gnext[c] - ny[2] - yh * ny[3]);
+            } else {
+                g[c] = gnext[c];
+            }
+        }
+        if (ln_in) fx.commit_ln(win, pre, gwin, bwin, nx_mean, nx_rstd);
+        else fx.commit(win, pre);
+    };
+    if (ln_in) lds_barrier();  // gamma and beta windows
     if (s0 + pl.slot < s1) {
-        fx.fetch(x + (s0 + pl.slot) * cells, pre);
-        load_cells<CPT>(dy + (s0 + pl.slot) * cells + pl.gc, g);
+        fetch_element(s0 + pl.slot);
+        take_element();
     }
     // Per element: commit its window, barrier, [stores of the PREVIOUS element], recompute,
     // reverse sweep, commit the next window.  The stores are issued one element late, away from
@@ -527,17 +679,12 @@ void step_bwd_fast(
         else store_cells<CPT>(dx + o, g_done);
         done_s = -1;
     };
-    if (s0 + pl.slot < s1) fx.commit(win, pre);
     for (int sb = s0; sb < s1; sb += NSLOT) {
         const int s = sb + pl.slot;
         const bool active = s < s1;  // a slot past the end idles through the barriers
         lds_barrier();               // this element's window
         finish_done();
-        float gnext[CPT];
-        if (s + NSLOT < s1) {
-            fx.fetch(x + (s + NSLOT) * cells, pre);
-            load_cells<CPT>(dy + (s + NSLOT) * cells + pl.gc, gnext);
-        }
+        if (s + NSLOT < s1) fetch_element(s + NSLOT);
         float cur[CPT];
         if (active) {
 #pragma unroll
@@ -605,10 +752,9 @@ void step_bwd_fast(
         for (int c = 0; c < CPT; ++c) {
             g_done[c] = g[c];
             d_done[c] = dsum[c];
-            g[c] = gnext[c];
         }
         // the x windows are free (the reverse sweep does not read them): commit the next one
-        if (s + NSLOT < s1) fx.commit(win, pre);
+        if (s + NSLOT < s1) take_element();
     }
     finish_done();
 
@@ -632,6 +778,10 @@ void step_bwd_fast(
         for (int c = 0; c < CPT; ++c) {
             reduce(db[c]);
             reduce(dr[c]);
+            if (LN) {
+                reduce(dgam[c]);
+                reduce(dbet[c]);
+            }
         }
         if (pl.slot != 0) return;
     }
@@ -645,6 +795,14 @@ void step_bwd_fast(
 #pragma unroll
     for (int c = 0; c < CPT; ++c) one[0][c] = dr[c];
     commit_grads<1, CPT>(dscale, one, param_mode, own_cell, always);
+    if (LN) {
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) one[0][c] = dgam[c];
+        commit_grads<1, CPT>(ln.dgamma, one, param_mode, own_cell, always);
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) one[0][c] = dbet[c];
+        commit_grads<1, CPT>(ln.dbeta, one, param_mode, own_cell, always);
+    }
 }
 
 // ---- backward, second kernel: everything that crosses a block boundary ----------------------
@@ -667,16 +825,25 @@ void step_bwd_fast(
 // A pass over one element is short (19 LDS reads, 18 FMAs per thread), and a block has few
 // workgroups to hide latency behind: a slot therefore takes E elements per round, so that
 // one barrier, one trip to LDS and one trip to memory serve E elements.
-template <int BS, int NSLOT, int E>
-__global__ __launch_bounds__((6 * BS * BS * NSLOT)) void step_bwd_cross(
+// LN (the LayerNorm of the network body folded in, see LnFold): when x is the raw output of the
+// step before, the x window holds xhat = (x - mean) * rstd and the affine part is applied as a
+// halo entry is used (its gamma and beta sit in registers beside the pair's weight).  dx as this
+// kernel completes it is the gradient with respect to LayerNorm(x): the row threads, which hold
+// the finished rows, also form the two per-sample sums that LayerNorm's backward needs,
+// sum(gamma dx) and sum(gamma dx xhat), and leave them per 16 lanes.
+template <int BS, int NSLOT, int E, bool LN>
+__global__ __launch_bounds__((6 * BS * BS * NSLOT)) __attribute__((amdgpu_waves_per_eu(3)))
+void step_bwd_cross(
     const float *__restrict__ weight, const float *__restrict__ x, const float *__restrict__ dsum,
     float *__restrict__ dweight, float *__restrict__ dx, int B, int M, int N, int K, int nblk,
-    int nchunk, int chunk_len, int param_mode) {
+    int nchunk, int chunk_len, int param_mode, LnFold ln) {
     using TL = Tile<BS, 1>;  // window geometry only
     constexpr int FS = BS * BS, TPS = 6 * FS;
     constexpr int PAIR = 2 * TL::WIN;              // [x window | D window] of one element
     constexpr int STAGE = E * PAIR;                // the E elements of a round
-    constexpr int SLOT = 2 * STAGE + 2 * E * TPS;  // two stages, two slabs
+    // two stages, two slabs; LN: two more slabs with xhat of the block's own cells, row by row
+    constexpr int XROWS = LN ? E * FS * BS : 0;
+    constexpr int SLOT = 2 * STAGE + 2 * E * TPS + 2 * XROWS;
     __shared__ __attribute__((aligned(16))) float lds[NSLOT * SLOT];
 
     int blk, chunk;
@@ -686,6 +853,7 @@ __global__ __launch_bounds__((6 * BS * BS * NSLOT)) void step_bwd_cross(
     const int p0 = (blk / (kb * nb)) * BS, q0 = ((blk / kb) % nb) * BS, r0 = (blk % kb) * BS;
     const FetchLines<TL, TPS> fx(lane, p0, q0, r0, M, N, K);
     float *stages = lds + slot * SLOT, *slabs = stages + 2 * STAGE;
+    float *xrows = slabs + 2 * E * TPS;
     const long cells = (long)M * N * K;
 
     // ---- which cell, which taps ----
@@ -705,7 +873,11 @@ __global__ __launch_bounds__((6 * BS * BS * NSLOT)) void step_bwd_cross(
     const long grow = ((long)(p0 + ri) * N + (q0 + rj)) * K + r0;
     const bool ri_edge = ri == 0 || ri == BS - 1, rj_edge = rj == 0 || rj == BS - 1;
 
+    const bool ln_in = LN && ln.x_stats != nullptr;
     float vx[9], cw[9];
+    float gh[9], bh[9];     // LN: gamma, beta of the pair's halo cell (1, 0 when x is used as is)
+    float grw[BS];  // LN, row threads: gamma of their row
+    if (ln_in && is_row) load_cells<BS>(ln.gamma + grow, grw);
     int hoff[9];
     bool mine[9];
 #pragma unroll
@@ -724,6 +896,10 @@ __global__ __launch_bounds__((6 * BS * BS * NSLOT)) void step_bwd_cross(
         hoff[pq] = own + di * TL::PS + dj * TL::RS + dk;
         const long hcell = gcell + (long)(di * N + dj) * K + dk;
         vx[pq] = (mine[pq] && in_grid) ? weight[(26 - t) * cells + hcell] : 0.f;
+        if (LN) {
+            gh[pq] = ln_in ? (in_grid ? ln.gamma[hcell] : 0.f) : 1.f;
+            bh[pq] = (ln_in && in_grid) ? ln.beta[hcell] : 0.f;
+        }
         // add-in-place mode: slot 0's accumulators start from what the gradient buffer holds
         cw[pq] = (mine[pq] && param_mode == kParamAddExclusive && slot == 0)
                      ? dweight[t * cells + gcell]
@@ -736,21 +912,25 @@ __global__ __launch_bounds__((6 * BS * BS * NSLOT)) void step_bwd_cross(
     // element e of round r of this slot; past the end of the chunk it is not `real`
     auto sample = [&](int r, int e) { return s0 + (r * E + e) * NSLOT + slot; };
     Buf px[E], pd[E];
+    float pmean[E], prstd[E];  // LN: statistics of the elements in px
     // Loads and commits are unconditional (past the end of the chunk they repeat its last
     // element, which nobody then uses): with branches around them the compiler cannot count the
     // loads in flight and waits for ALL of them wherever it needs one.
     auto fetch_round = [&](int r) {
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            const long at = (long)min(sample(r, e), s1 - 1) * cells;
+            const int sc = min(sample(r, e), s1 - 1);
+            const long at = (long)sc * cells;
             fx.fetch(x + at, px[e]);
             fx.fetch(dsum + at, pd[e]);
+            pmean[e] = ln_in ? load_ahead(ln.x_stats, 2 * sc) : 0.f;
+            prstd[e] = ln_in ? load_ahead(ln.x_stats, 2 * sc + 1) : 1.f;
         }
     };
     auto commit_round = [&](int st) {
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            fx.template commit<1>(stages + st * STAGE + e * PAIR, px[e]);
+            fx.template commit<1>(stages + st * STAGE + e * PAIR, px[e], pmean[e], prstd[e]);
             fx.template commit<1>(stages + st * STAGE + e * PAIR + TL::WIN, pd[e]);
         }
     };
@@ -779,6 +959,23 @@ __global__ __launch_bounds__((6 * BS * BS * NSLOT)) void step_bwd_cross(
                     for (int c = 0; c < BS; ++c) gx[e][c] += part[c];
                 }
                 if (s < s1) store_cells<BS>(dx + (long)s * cells + grow, gx[e]);
+                if (ln_in) {
+                    float xh[BS], t1 = 0.f, t2 = 0.f;
+                    load_cells<BS>(xrows + (st * E + e) * FS * BS + lane * BS, xh);
+#pragma unroll
+                    for (int c = 0; c < BS; ++c) {
+                        const float a = grw[c] * gx[e][c];
+                        t1 += a;
+                        t2 = fmaf(a, xh[c], t2);
+                    }
+                    t1 = row16_sum(t1);  // the row threads are whole 16-lane groups
+                    t2 = row16_sum(t2);
+                    if ((lane & 15) == 0 && s < s1) {
+                        float *to = ln.x_part + (((long)s * nblk + blk) * (FS / 16) + lane / 16) * 2;
+                        to[0] = t1;
+                        to[1] = t2;
+                    }
+                }
             }
         }
         r_prev = -1;
@@ -811,9 +1008,15 @@ __global__ __launch_bounds__((6 * BS * BS * NSLOT)) void step_bwd_cross(
 #pragma unroll
             for (int pq = 0; pq < 9; ++pq) {
                 g = fmaf(vx[pq], dh[pq], g);
-                cw[pq] = fmaf(real ? dc : 0.f, xh[pq], cw[pq]);
+                cw[pq] = fmaf(real ? dc : 0.f, LN ? fmaf(xh[pq], gh[pq], bh[pq]) : xh[pq], cw[pq]);
             }
             slabs[(st * E + e) * TPS + lane] = g;
+            if (ln_in && is_row) {  // xhat of the own row, for the sums one round later
+                float xr[BS];
+#pragma unroll
+                for (int c = 0; c < BS; ++c) xr[c] = xw[(ri + 1) * TL::PS + (rj + 1) * TL::RS + 1 + c];
+                store_cells<BS>(xrows + (st * E + e) * FS * BS + lane * BS, xr);
+            }
         }
         r_prev = r;
         commit_round(st ^ 1);
@@ -899,9 +1102,9 @@ Plan make_plan(const StepArgs &a, int nslot, int resident, bool whole_batch_per_
     return p;
 }
 
-template <int BS, int CPT, int NSLOT, int ACT> int launch_fwd(const StepArgs &a, hipStream_t st) {
+template <int BS, int CPT, int NSLOT, int ACT, bool LN> int launch_fwd_ln(const StepArgs &a, hipStream_t st) {
     using TL = Tile<BS, CPT>;
-    auto kern = step_fwd_fast<BS, CPT, NSLOT, ACT>;
+    auto kern = step_fwd_fast<BS, CPT, NSLOT, ACT, LN>;
     static int per_cu = 0;
     if (per_cu == 0) {
         int n = 0;
@@ -914,8 +1117,12 @@ template <int BS, int CPT, int NSLOT, int ACT> int launch_fwd(const StepArgs &a,
     hipLaunchKernelGGL(kern, dim3(padded_grid(p.nblk, p.nchunk)), dim3(TL::TPS * NSLOT), 0, st,
                        (const float *)a.weight, (const float *)a.bias, (const float *)a.scale,
                        (const float *)a.x, (float *)a.y, a.B, a.M, a.N, a.K, a.inner, p.nblk, p.nchunk,
-                       p.chunk_len);
+                       p.chunk_len, a.ln);
     return check_launch("step_fwd_fast");
+}
+template <int BS, int CPT, int NSLOT, int ACT> int launch_fwd(const StepArgs &a, hipStream_t st) {
+    if (a.ln.gamma) return launch_fwd_ln<BS, CPT, NSLOT, ACT, true>(a, st);
+    return launch_fwd_ln<BS, CPT, NSLOT, ACT, false>(a, st);
 }
 
 constexpr size_t kMaxLds = 160 * 1024;
@@ -924,11 +1131,12 @@ constexpr size_t kMaxLds = 160 * 1024;
 constexpr int kCrossSlots8 = 1, kCrossElems8 = 2;  // bs=8: 384 threads, one wave per face
 constexpr int kCrossSlots4 = 4, kCrossElems4 = 2;  // bs=4: four slots of 96 threads
 
-template <int BS, int CPT, int NSLOT, int ACT> int launch_bwd(const StepArgs &a, hipStream_t st) {
+template <int BS, int CPT, int NSLOT, int ACT, bool LN>
+int launch_bwd_ln(const StepArgs &a, hipStream_t st) {
     using TL = Tile<BS, CPT>;
     const long cells = (long)a.M * a.N * a.K;
-    const size_t lds = bwd_lds_bytes<BS, CPT, NSLOT>(a.inner);
-    auto kern = step_bwd_fast<BS, CPT, NSLOT, ACT>;
+    const size_t lds = bwd_lds_bytes<BS, CPT, NSLOT>(a.inner) + (LN ? 2 * TL::WIN * sizeof(float) : 0);
+    auto kern = step_bwd_fast<BS, CPT, NSLOT, ACT, LN>;
     static bool big_lds_enabled = false;            // per instantiation
     static int per_cu_cache[kMaxBackwardIters + 1];  // per instantiation, by inner iterations
     if (lds > 64 * 1024 && !big_lds_enabled) {
@@ -960,24 +1168,33 @@ template <int BS, int CPT, int NSLOT, int ACT> int launch_bwd(const StepArgs &a,
         if (int rc = fill_zero((float *)a.dweight, 27 * cells, st)) return rc;
         if (int rc = fill_zero((float *)a.dbias, cells, st)) return rc;
         if (int rc = fill_zero((float *)a.dscale, cells, st)) return rc;
+        if (LN) {
+            if (int rc = fill_zero(a.ln.dgamma, cells, st)) return rc;
+            if (int rc = fill_zero(a.ln.dbeta, cells, st)) return rc;
+        }
     }
     const int dx_accumulate = (a.flags & GRIDNET_OVERWRITE_DX) ? 0 : 1;
     hipLaunchKernelGGL(kern, dim3(padded_grid(p.nblk, p.nchunk)), dim3(TL::TPS * NSLOT), lds, st,
                        (const float *)a.weight, (const float *)a.bias, (const float *)a.scale,
                        (const float *)a.x, (const float *)a.dy, (float *)a.dweight, (float *)a.dbias,
                        (float *)a.dscale, (float *)a.dx, (float *)a.workspace, a.B, a.M, a.N, a.K,
-                       a.inner, p.nblk, p.nchunk, p.chunk_len, param_mode, dx_accumulate);
+                       a.inner, p.nblk, p.nchunk, p.chunk_len, param_mode, dx_accumulate, a.ln);
     if (int rc = check_launch("step_bwd_fast")) return rc;
     // same blocks, same batch chunks, same way of committing parameter gradients (the two
     // kernels write disjoint entries of dweight)
     constexpr int XSLOT = BS == 8 ? kCrossSlots8 : kCrossSlots4;
     constexpr int XE = BS == 8 ? kCrossElems8 : kCrossElems4;
-    hipLaunchKernelGGL((step_bwd_cross<BS, XSLOT, XE>), dim3(padded_grid(p.nblk, p.nchunk)),
+    hipLaunchKernelGGL((step_bwd_cross<BS, XSLOT, XE, LN>), dim3(padded_grid(p.nblk, p.nchunk)),
                        dim3(6 * BS * BS * XSLOT), 0, st, (const float *)a.weight,
                        (const float *)a.x, (const float *)a.workspace, (float *)a.dweight,
-                       (float *)a.dx, a.B, a.M, a.N, a.K, p.nblk, p.nchunk, p.chunk_len, param_mode);
+                       (float *)a.dx, a.B, a.M, a.N, a.K, p.nblk, p.nchunk, p.chunk_len, param_mode,
+                       a.ln);
     if (int rc = check_launch("step_bwd_cross")) return rc;
     return GRIDNET_OK;
+}
+template <int BS, int CPT, int NSLOT, int ACT> int launch_bwd(const StepArgs &a, hipStream_t st) {
+    if (a.ln.gamma) return launch_bwd_ln<BS, CPT, NSLOT, ACT, true>(a, st);
+    return launch_bwd_ln<BS, CPT, NSLOT, ACT, false>(a, st);
 }
 
 // ---- the tuned shapes ---------------------------------------------------------------------
@@ -1007,12 +1224,19 @@ template <bool BWD> int dispatch(const StepArgs &a, hipStream_t st) {
 
 }  // namespace
 
+int step_fast_forward_parts(int block_size) {
+    return block_size == 8 ? Tile<8, kFwdCpt8>::TPS / 16 : Tile<4, kFwdCpt4>::TPS / 16;
+}
+int step_fast_forward_part_count(int block_size) { return 16 * (block_size == 8 ? kFwdCpt8 : kFwdCpt4); }
+int step_fast_backward_parts(int block_size) { return block_size * block_size / 16; }
+
 bool step_fast_supports(const StepArgs &a, bool backward) {
     if (a.dtype != GRIDNET_F32 || a.normalize) return false;
     if (a.block_size != 4 && a.block_size != 8) return false;
     if (backward) {
-        const size_t lds = a.block_size == 8 ? bwd_lds_bytes<8, kBwdCpt8, kBwdSlots8>(a.inner)
-                                             : bwd_lds_bytes<4, kBwdCpt4, kBwdSlots4>(a.inner);
+        size_t lds = a.block_size == 8 ? bwd_lds_bytes<8, kBwdCpt8, kBwdSlots8>(a.inner)
+                                       : bwd_lds_bytes<4, kBwdCpt4, kBwdSlots4>(a.inner);
+        if (a.ln.gamma) lds += 2 * (a.block_size == 8 ? Tile<8, 1>::WIN : Tile<4, 1>::WIN) * sizeof(float);
         if (lds > kMaxLds) return false;
     }
     return true;

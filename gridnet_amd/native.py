@@ -32,6 +32,11 @@ EXPORTS = (
     "gridnet_hip_layernorm_workspace_bytes",
     "gridnet_hip_layernorm_forward",
     "gridnet_hip_layernorm_backward",
+    "gridnet_hip_fused_workspace_bytes",
+    "gridnet_hip_fused_forward",
+    "gridnet_hip_layernorm_apply",
+    "gridnet_hip_layernorm_backward_sums",
+    "gridnet_hip_fused_backward",
 )
 
 
@@ -69,6 +74,17 @@ def _load():
     lib.gridnet_hip_layernorm_forward.argtypes = [i, p, p, p, p, p, p, i, l, d, p, z, p]
     lib.gridnet_hip_layernorm_backward.restype = i
     lib.gridnet_hip_layernorm_backward.argtypes = [i, p, p, p, p, p, p, p, p, i, l, i, p, z, p]
+    lib.gridnet_hip_fused_workspace_bytes.restype = z
+    lib.gridnet_hip_fused_workspace_bytes.argtypes = [i, i, i, i, i, i, i]
+    lib.gridnet_hip_fused_forward.restype = i
+    lib.gridnet_hip_fused_forward.argtypes = [i, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, d, i,
+                                              p, z, p]
+    lib.gridnet_hip_layernorm_apply.restype = i
+    lib.gridnet_hip_layernorm_apply.argtypes = [i, p, p, p, p, p, i, l, p]
+    lib.gridnet_hip_layernorm_backward_sums.restype = i
+    lib.gridnet_hip_layernorm_backward_sums.argtypes = [i, p, p, p, p, p, i, l, p, z, p]
+    lib.gridnet_hip_fused_backward.restype = i
+    lib.gridnet_hip_fused_backward.argtypes = [i] + [p] * 18 + [i] * 8 + [p, z, p]
     return lib
 
 

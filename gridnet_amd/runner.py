@@ -4,6 +4,11 @@ forward, then the same chain backward, on preallocated buffers.
 This is what a training loop that owns its buffers (or a captured HIP graph) calls; the
 autograd ops in ``backend_cuda``/``layernorm`` do the same launches with torch-managed
 memory.  Order of operations: gridnet/scripts/train_mnist.py:62-64.
+
+``fused=True`` runs the same chain through the entry points that fold the LayerNorm into the
+step kernels: a step reads the raw output of the step before it and normalises it while
+loading, so the LayerNorm costs no pass over the activations of its own (one, for the final
+output).  Same results within rounding; fp32, ``normalize=False``, ``inner >= 1`` only.
 """
 
 import torch
@@ -14,7 +19,8 @@ from . import native as _n
 class BodyRunner:
     def __init__(self, weight, bias, scale, gamma, beta, batch: int, inner: int, outer: int,
                  block_size: int, activation: str = "leaky_relu", normalize: bool = False,
-                 eps: float = 1e-5, ln_eps: float = 1e-5, backward: bool = True):
+                 eps: float = 1e-5, ln_eps: float = 1e-5, backward: bool = True,
+                 fused: bool = False):
         self.w, self.b, self.r, self.gamma, self.beta = weight, bias, scale, gamma, beta
         self.B, (self.M, self.N, self.K) = batch, bias.shape
         self.inner, self.outer, self.bs = inner, outer, block_size
@@ -46,6 +52,19 @@ class BodyRunner:
                 self.dt, batch, self.M, self.N, self.K, inner, block_size, self.normalize)
             self.bw_ws = _n.workspace(self.bw_ws_bytes, dev)
         self.on_launch = None  # optional hook(name, phase) for per-kernel timing
+        self.fused = fused
+        if fused:
+            if weight.dtype != torch.float32 or normalize or inner < 1:
+                raise RuntimeError("the fused body covers float32, normalize=False, inner >= 1")
+            self.stats = torch.empty(max(keep, 2), batch, 2, device=dev, dtype=dtype)
+            self.fw_ws_bytes = _n.lib.gridnet_hip_fused_workspace_bytes(
+                batch, self.M, self.N, self.K, inner, block_size, 0)
+            self.fw_ws = _n.workspace(self.fw_ws_bytes, dev)
+            if backward:
+                self.sums = torch.empty(keep, batch, 2, device=dev, dtype=dtype)
+                self.fb_ws_bytes = _n.lib.gridnet_hip_fused_workspace_bytes(
+                    batch, self.M, self.N, self.K, inner, block_size, 1)
+                self.fb_ws = _n.workspace(self.fb_ws_bytes, dev)
 
     def _mark(self, name, phase):
         if self.on_launch is not None:
@@ -67,8 +86,65 @@ class BodyRunner:
             self.ln_ws.data_ptr(), self.ln_ws_bytes, stream))
         self._mark("ln_fwd", 1)
 
+    # ---- the fused chain: s[j] = raw output of step j, stats[j] = its LayerNorm statistics ----
+    def _fused_forward(self, x0):
+        stream = _n.current_stream(self.w)
+        keep = self.has_backward
+        self.x0 = x0
+        x, x_stats = x0, None
+        for j in range(self.outer):
+            # forward only: nothing is kept, two raw buffers and two statistics rows alternate
+            y = self.s[j] if keep else (self.s[0], self.h[1])[j % 2]
+            y_stats = self.stats[j if keep else j % 2]
+            self._mark("step_fwd", 0)
+            _n.check(_n.lib.gridnet_hip_fused_forward(
+                self.dt, self.w.data_ptr(), self.b.data_ptr(), self.r.data_ptr(),
+                self.gamma.data_ptr(), self.beta.data_ptr(), x.data_ptr(),
+                x_stats.data_ptr() if x_stats is not None else None, y.data_ptr(),
+                y_stats.data_ptr(), self.B, self.M, self.N, self.K, self.inner, self.bs,
+                self.ln_eps, self.act, self.fw_ws.data_ptr(), self.fw_ws_bytes, stream))
+            self._mark("step_fwd", 1)
+            x, x_stats = y, y_stats
+        out = self.h[0]
+        self._mark("ln_fwd", 0)
+        _n.check(_n.lib.gridnet_hip_layernorm_apply(
+            self.dt, x.data_ptr(), x_stats.data_ptr(), self.gamma.data_ptr(), self.beta.data_ptr(),
+            out.data_ptr(), self.B, self.n, stream))
+        self._mark("ln_fwd", 1)
+        return out
+
+    def _fused_backward(self, grad_out):
+        stream = _n.current_stream(self.w)
+        last = self.outer - 1
+        self._mark("ln_bwd", 0)
+        _n.check(_n.lib.gridnet_hip_layernorm_backward_sums(
+            self.dt, grad_out.data_ptr(), self.s[last].data_ptr(), self.stats[last].data_ptr(),
+            self.gamma.data_ptr(), self.sums[last].data_ptr(), self.B, self.n,
+            self.ln_ws.data_ptr(), self.ln_ws_bytes, stream))
+        self._mark("ln_bwd", 1)
+        g = grad_out
+        for j in reversed(range(self.outer)):
+            x = self.s[j - 1] if j else self.x0
+            dst = self.ga if g is not self.ga else self.gb
+            self._mark("step_bwd", 0)
+            _n.check(_n.lib.gridnet_hip_fused_backward(
+                self.dt, self.w.data_ptr(), self.b.data_ptr(), self.r.data_ptr(),
+                self.gamma.data_ptr(), self.beta.data_ptr(), x.data_ptr(),
+                self.stats[j - 1].data_ptr() if j else None, g.data_ptr(), self.s[j].data_ptr(),
+                self.stats[j].data_ptr(), self.sums[j].data_ptr(), self.dw.data_ptr(),
+                self.db.data_ptr(), self.dr.data_ptr(), self.dgamma.data_ptr(),
+                self.dbeta.data_ptr(), dst.data_ptr(), self.sums[j - 1].data_ptr() if j else None,
+                self.B, self.M, self.N, self.K, self.inner, self.bs, self.act,
+                _n.OVERWRITE_PARAMS if j == last else 0, self.fb_ws.data_ptr(), self.fb_ws_bytes,
+                stream))
+            self._mark("step_bwd", 1)
+            g = dst
+        return self.dw, self.db, self.dr, self.dgamma, self.dbeta, g
+
     def forward(self, x0):
         """Returns the buffer holding the result (valid until the next call)."""
+        if self.fused:
+            return self._fused_forward(x0)
         stream = _n.current_stream(self.w)
         self.h[0].copy_(x0)
         if self.has_backward:
@@ -85,6 +161,8 @@ class BodyRunner:
         """Backward of the last ``forward``.  Returns (dweight, dbias, dscale, dgamma, dbeta, dx0);
         parameter gradients are summed over the outer steps (shared parameters)."""
         assert self.has_backward
+        if self.fused:
+            return self._fused_backward(grad_out)
         stream = _n.current_stream(self.w)
         g = grad_out
         for j in reversed(range(self.outer)):

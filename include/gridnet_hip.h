@@ -132,6 +132,57 @@ int gridnet_hip_layernorm_backward(int dtype, const void *dy, const void *x, con
                                    void *dbeta, int B, long n, int flags, void *workspace,
                                    size_t workspace_bytes, void *stream);
 
+/*
+ * ---- The network body with the LayerNorm folded into the step kernels ----------------------
+ * The reference's callers run `h = norm(net(h))` op by op, `outer` times
+ * (gridnet/scripts/train_mnist.py:62-64, gridnet/scripts/train_imagenet.py:76-86); these entry
+ * points compute the same chain without a pass over the activations for each LayerNorm: a step
+ * reads the RAW output of the step before it and normalises it while loading, and leaves its own
+ * raw output together with that output's LayerNorm statistics.  They have no counterpart in the
+ * reference's extension; results agree with the op-by-op chain to rounding.
+ *
+ * float32, normalize = false, inner >= 1, block_size in {4, 8}; other problems are rejected with
+ * GRIDNET_ERR_ARGUMENT (use the step and LayerNorm entry points above).
+ *   stats  [B, 2]: (mean, rstd) of a LayerNorm over one sample's M*N*K cells
+ *   sums   [B, 2]: the two per-sample means its backward needs, mean(gamma*g) and
+ *                  mean(gamma*g*xhat), g the gradient with respect to the LayerNorm's output
+ */
+size_t gridnet_hip_fused_workspace_bytes(int B, int M, int N, int K, int inner, int block_size,
+                                         int backward);
+
+/* y_raw = step(LayerNorm(x; x_stats, gamma, beta)), y_stats = statistics of y_raw.
+ * x_stats == NULL: x is used as it is (the first step of a chain). */
+int gridnet_hip_fused_forward(int dtype, const void *weight, const void *bias, const void *scale,
+                              const void *gamma, const void *beta, const void *x,
+                              const void *x_stats, void *y_raw, void *y_stats, int B, int M, int N,
+                              int K, int inner, int block_size, double ln_eps, int activation,
+                              void *workspace, size_t workspace_bytes, void *stream);
+
+/* y = (x - mean) * rstd * gamma + beta with statistics that are already known: the LayerNorm
+ * after the LAST step of a chain, whose output is needed as a tensor. */
+int gridnet_hip_layernorm_apply(int dtype, const void *x, const void *stats, const void *gamma,
+                                const void *beta, void *y, int B, long n, void *stream);
+
+/* `sums` of a LayerNorm from the gradient dy with respect to its output: what the backward of a
+ * chain starts from.  workspace: gridnet_hip_layernorm_workspace_bytes(). */
+int gridnet_hip_layernorm_backward_sums(int dtype, const void *dy, const void *x, const void *stats,
+                                        const void *gamma, void *sums, int B, long n,
+                                        void *workspace, size_t workspace_bytes, void *stream);
+
+/* Backward of gridnet_hip_fused_forward.  dy is the gradient with respect to
+ * LayerNorm(y_raw; y_stats); y_sums are that LayerNorm's sums.  dweight, dbias, dscale, dgamma,
+ * dbeta (dgamma, dbeta: of the LayerNorm after this step) are accumulated, or written with
+ * GRIDNET_OVERWRITE_PARAMS.  dx is always fully written: the gradient with respect to
+ * LayerNorm(x; x_stats) -- the dy of the step before -- and x_sums receives its sums; with
+ * x_stats == NULL (first step) dx is the gradient with respect to x and x_sums must be NULL. */
+int gridnet_hip_fused_backward(int dtype, const void *weight, const void *bias, const void *scale,
+                               const void *gamma, const void *beta, const void *x,
+                               const void *x_stats, const void *dy, const void *y_raw,
+                               const void *y_stats, const void *y_sums, void *dweight, void *dbias,
+                               void *dscale, void *dgamma, void *dbeta, void *dx, void *x_sums, int B,
+                               int M, int N, int K, int inner, int block_size, int activation,
+                               int flags, void *workspace, size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,143 @@
+"""GPU parity of the entry points that fold the LayerNorm into the step kernels
+(gridnet_hip_fused_forward / _backward and the LayerNorm pieces beside them): the whole chain
+outer x (step, LayerNorm), forward and backward, against the CPU oracle (fp64 evaluation of the
+reference's op sequence, gridnet/scripts/train_imagenet.py:76-86) and against the op-by-op
+chain of the same library.  Bar: rtol 1e-4 / atol 1e-5."""
+
+import dataclasses
+
+import pytest
+import torch
+
+from oracle.network import network_forward, network_forward_backward
+
+from helpers import assert_close
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+PARAMS = ("weight", "bias", "scale", "gamma", "beta")
+NAMES = ("y", "dweight", "dbias", "dscale", "dgamma", "dbeta", "dx0")
+
+
+def runner_for(wl, t, backward, fused):
+    from gridnet_amd.runner import BodyRunner
+
+    d = {k: v.to(DEV) for k, v in t.items()}
+    run = BodyRunner(d["weight"], d["bias"], d["scale"], d["gamma"], d["beta"], t["x0"].shape[0],
+                     wl.inner, wl.outer, wl.block_size, wl.activation, wl.normalize,
+                     backward=backward, fused=fused)
+    return run, d
+
+
+def randomise_affine(t, seed=7):
+    """gamma = 1, beta = 0 would hide a mix-up of the two, or of which cell's pair is used."""
+    g = torch.Generator().manual_seed(seed)
+    t["gamma"] = 1 + 0.2 * torch.randn(t["gamma"].shape, generator=g)
+    t["beta"] = 0.2 * torch.randn(t["beta"].shape, generator=g)
+    return t
+
+
+def run_fused(wl, t, backward):
+    run, d = runner_for(wl, t, backward, True)
+    y = run.forward(d["x0"]).clone()
+    if not backward:
+        return (y,)
+    return (y, *[g.clone() for g in run.backward(d["grad_out"])])
+
+
+def oracle(wl, t, backward):
+    if not backward:
+        return (network_forward(*[t[k].double() for k in PARAMS], t["x0"].double(), wl.inner,
+                                wl.outer, wl.block_size, wl.activation, wl.normalize),)
+    return network_forward_backward(
+        [t[k].double() for k in PARAMS], t["x0"].double(), t["grad_out"].double(),
+        inner_iterations=wl.inner, outer_iterations=wl.outer, block_size=wl.block_size,
+        activation=wl.activation, normalize=wl.normalize)
+
+
+@pytest.mark.parametrize("name,grid,batch,outer", [("C1", 16, 2, 2), ("C3", 32, 3, 3),
+                                                   ("C5", 16, 5, 3), ("C3", 16, 1, 1)])
+def test_fused_chain_matches_oracle(name, grid, batch, outer):
+    from gridnet_amd.configs import WORKLOADS, make_inputs
+
+    wl = dataclasses.replace(WORKLOADS[name], grid=grid, batch=batch, outer=outer, backward=True)
+    print(f"fused {wl.name} grid={grid} batch={batch} outer={outer}", flush=True)
+    t = randomise_affine(make_inputs(wl))
+    if wl.inner >= 8:  # keep 8 residual updates contractive (fp32 rounding otherwise grows)
+        t["weight"], t["scale"] = t["weight"] * 0.5, t["scale"] * 0.5
+    for name_, got, exp in zip(NAMES, run_fused(wl, t, True), oracle(wl, t, True)):
+        assert_close(got, exp, what=name_)
+
+
+@pytest.mark.parametrize("name,grid,batch,outer", [("C2", 32, 4, 3), ("C4", 32, 2, 2)])
+def test_fused_forward_only_matches_oracle(name, grid, batch, outer):
+    from gridnet_amd.configs import WORKLOADS, make_inputs
+
+    wl = dataclasses.replace(WORKLOADS[name], grid=grid, batch=batch, outer=outer)
+    print(f"fused forward {wl.name} grid={grid} batch={batch} outer={outer}", flush=True)
+    t = randomise_affine(make_inputs(wl))
+    (got,), (exp,) = run_fused(wl, t, False), oracle(wl, t, False)
+    assert_close(got, exp, what="y")
+
+
+@pytest.mark.parametrize("shape", [(8, 16, 24), (24, 8, 16)])
+def test_fused_chain_non_cubic_grid(shape):
+    """Axes of different lengths: catches a swapped stride in the window, face or row indexing."""
+    from gridnet_amd.runner import BodyRunner
+    from helpers import make_acts, make_params
+
+    inner, outer, bs, batch = 2, 2, 8, 3
+    print(f"fused non-cubic shape={shape}", flush=True)
+    w, b, r = make_params(shape, seed=21)
+    g = torch.Generator().manual_seed(3)
+    gamma = 1 + 0.2 * torch.randn(shape, generator=g)
+    beta = 0.2 * torch.randn(shape, generator=g)
+    x0, gy = make_acts(batch, shape, seed=22), make_acts(batch, shape, seed=23)
+    run = BodyRunner(*(v.to(DEV) for v in (w, b, r, gamma, beta)), batch, inner, outer, bs,
+                     "silu", False, backward=True, fused=True)
+    y = run.forward(x0.to(DEV)).clone()
+    got = (y, *[v.clone() for v in run.backward(gy.to(DEV))])
+    exp = network_forward_backward([v.double() for v in (w, b, r, gamma, beta)], x0.double(),
+                                   gy.double(), inner_iterations=inner, outer_iterations=outer,
+                                   block_size=bs, activation="silu", normalize=False)
+    for name_, a, e in zip(NAMES, got, exp):
+        assert_close(a, e, what=name_)
+
+
+def test_fused_full_size_agrees_with_op_by_op_chain():
+    """The graded shape (64^3 grid, 8^3 blocks, inner 4) at full size, where the oracle is too
+    slow: the fused chain against the op-by-op chain of the same library (itself checked against
+    the oracle on smaller shapes; twice the bar, see below), and bitwise reproducibility of the
+    fused chain."""
+    from gridnet_amd.configs import WORKLOADS, make_inputs
+
+    wl = dataclasses.replace(WORKLOADS["C3"], batch=4, outer=3)
+    t = randomise_affine(make_inputs(wl))
+    print(f"fused vs op-by-op {wl.name} batch=4 outer=3", flush=True)
+    run_s, d = runner_for(wl, t, True, False)
+    ys = run_s.forward(d["x0"]).clone()
+    gs = [g.clone() for g in run_s.backward(d["grad_out"])]
+    first = run_fused(wl, t, True)
+    # two fp32 evaluations in different orders, each within the bar of the exact result:
+    # twice the bar between them
+    for name_, a, e in zip(NAMES, first, (ys, *gs)):
+        assert_close(a, e.double().cpu(), rtol=2e-4, atol=2e-5, what=name_)
+    again = run_fused(wl, t, True)
+    for name_, a, e in zip(NAMES, again, first):
+        assert torch.equal(a, e), f"{name_}: fused chain is not bitwise reproducible"
+
+
+def test_fused_rejects_what_it_does_not_cover():
+    from gridnet_amd import native as n
+
+    x = torch.zeros(1, 8, 8, 8, device=DEV, dtype=torch.float64)
+    p = x.data_ptr()
+    rc = n.lib.gridnet_hip_fused_forward(n.F64, p, p, p, p, p, p, None, p, p, 1, 8, 8, 8, 1, 8, 1e-5,
+                                         0, p, 1 << 20, n.current_stream(x))
+    assert rc != 0 and "float32" in n.last_error()
+    rc = n.lib.gridnet_hip_fused_forward(n.F32, p, p, p, p, p, p, None, p, p, 1, 8, 8, 8, 0, 8, 1e-5,
+                                         0, p, 1 << 20, n.current_stream(x))
+    assert rc != 0 and "inner" in n.last_error()
+    rc = n.lib.gridnet_hip_fused_forward(n.F32, p, p, p, p, p, p, None, p, p, 1, 8, 8, 8, 1, 8, 1e-5,
+                                         0, p, 0, n.current_stream(x))
+    assert rc != 0 and "workspace" in n.last_error()
