@@ -10,10 +10,12 @@
 //                                fixed order (exact pairwise-combination formula, no
 //                                E[x^2]-mean^2 cancellation) and normalises its chunk
 //   backward  ln_bwd_partial   : per chunk sum(g) and sum(g*xhat), g = dy*gamma
-//             ln_bwd_finalize  : per sample means of the two
-//             ln_bwd_apply     : one thread owns 4 adjacent cells for ALL samples, so dgamma
-//                                and dbeta are reduced over the batch in registers, without
-//                                atomics and in a fixed order
+//             ln_bwd_apply     : every workgroup merges the chunk sums into the per-sample
+//                                means; one thread owns 4 adjacent cells for ALL samples, so
+//                                dgamma and dbeta are reduced over the batch in registers,
+//                                without atomics and in a fixed order
+//             (ln_bwd_finalize : the per-sample means as a kernel of their own, for the
+//                                callers that need them as a tensor)
 //
 // Every reduction has a fixed order, so results are bitwise reproducible.
 
@@ -196,37 +198,69 @@ __global__ __launch_bounds__(kLnThreads) void ln_bwd_finalize(const T *__restric
     }
 }
 
+// The per-sample means of the two sums are formed here, by every workgroup for itself, from the
+// chunk partials (8 lanes per sample, fixed order): B * nchunk pairs are little to read next to
+// the B * 1024 * VEC cells a workgroup streams, and a kernel of its own for it costs more in
+// launch and drain than it computes.  Samples are handled kLnSumBatch at a time.
+constexpr int kLnSumBatch = kLnThreads / 8;
+
 template <typename T, int VEC, bool ACCUM>
 __global__ __launch_bounds__(kLnThreads) void ln_bwd_apply(
     const T *__restrict__ dy, const T *__restrict__ x, const T *__restrict__ gamma,
-    const T *__restrict__ mean, const T *__restrict__ rstd, const T *__restrict__ sample_means,
-    T *__restrict__ dx, T *__restrict__ dgamma, T *__restrict__ dbeta, int B, long n) {
+    const T *__restrict__ mean, const T *__restrict__ rstd, const T *__restrict__ partial,
+    int nchunk, T *__restrict__ dx, T *__restrict__ dgamma, T *__restrict__ dbeta, int B, long n) {
+    __shared__ T sample_means[kLnSumBatch * 2];
     const long at = ((long)blockIdx.x * kLnThreads + threadIdx.x) * VEC;
-    if (at >= n) return;
+    const bool live = at < n;
     T gm[VEC], dg[VEC], dbt[VEC];
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
-        gm[e] = gamma[at + e];
+        gm[e] = live ? gamma[at + e] : T(0);
         dg[e] = T(0);
         dbt[e] = T(0);
     }
     struct alignas(sizeof(T) * VEC) Pack { T v[VEC]; };
-#pragma unroll 4
-    for (int b = 0; b < B; ++b) {
-        const T mu = mean[b], rs = rstd[b];
-        const T c1 = sample_means[b * 2], c2 = sample_means[b * 2 + 1];
-        const Pack d = *reinterpret_cast<const Pack *>(dy + (long)b * n + at);
-        const Pack xv = *reinterpret_cast<const Pack *>(x + (long)b * n + at);
-        Pack o;
+    for (int b0 = 0; b0 < B; b0 += kLnSumBatch) {
+        {   // means of the next kLnSumBatch samples: lane group of 8 per sample
+            const int sb = b0 + threadIdx.x / 8, part = threadIdx.x % 8;
+            T s1 = T(0), s2 = T(0);
+            if (sb < B)
+                for (int c = part; c < nchunk; c += 8) {
+                    s1 += partial[((long)sb * nchunk + c) * 2];
+                    s2 += partial[((long)sb * nchunk + c) * 2 + 1];
+                }
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-            const T xh = (xv.v[e] - mu) * rs;
-            dg[e] += d.v[e] * xh;
-            dbt[e] += d.v[e];
-            o.v[e] = rs * (d.v[e] * gm[e] - c1 - xh * c2);
+            for (int off = 4; off > 0; off >>= 1) {
+                s1 += __shfl_xor(s1, off, 8);
+                s2 += __shfl_xor(s2, off, 8);
+            }
+            __syncthreads();  // the previous batch's values are no longer read
+            if (part == 0) {
+                sample_means[(threadIdx.x / 8) * 2] = s1 / T(n);
+                sample_means[(threadIdx.x / 8) * 2 + 1] = s2 / T(n);
+            }
+            __syncthreads();
         }
-        *reinterpret_cast<Pack *>(dx + (long)b * n + at) = o;
+        if (!live) continue;
+        const int bend = min(B, b0 + kLnSumBatch);
+#pragma unroll 4
+        for (int b = b0; b < bend; ++b) {
+            const T mu = mean[b], rs = rstd[b];
+            const T c1 = sample_means[(b - b0) * 2], c2 = sample_means[(b - b0) * 2 + 1];
+            const Pack d = *reinterpret_cast<const Pack *>(dy + (long)b * n + at);
+            const Pack xv = *reinterpret_cast<const Pack *>(x + (long)b * n + at);
+            Pack o;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) {
+                const T xh = (xv.v[e] - mu) * rs;
+                dg[e] += d.v[e] * xh;
+                dbt[e] += d.v[e];
+                o.v[e] = rs * (d.v[e] * gm[e] - c1 - xh * c2);
+            }
+            *reinterpret_cast<Pack *>(dx + (long)b * n + at) = o;
+        }
     }
+    if (!live) return;
 #pragma unroll
     for (int e = 0; e < VEC; ++e) {
         if (ACCUM) {
@@ -360,7 +394,6 @@ template <typename T> int forward_t(const LayerNormArgs &a, hipStream_t st) {
 template <typename T> int backward_t(const LayerNormArgs &a, hipStream_t st) {
     const int nchunk = chunks_of(a.n);
     T *partial = (T *)a.workspace;
-    T *sample_means = partial + (long)a.B * nchunk * 2;
     const bool vec = a.n % 4 == 0 && aligned4<T>(a.x) && aligned4<T>(a.dy) && aligned4<T>(a.gamma) &&
                      aligned4<T>(a.dx);
     const bool accum = (a.flags & GRIDNET_OVERWRITE_PARAMS) == 0;
@@ -373,13 +406,11 @@ template <typename T> int backward_t(const LayerNormArgs &a, hipStream_t st) {
         hipLaunchKernelGGL((ln_bwd_partial<T, false>), grid, block, 0, st, (const T *)a.dy,
                            (const T *)a.x, (const T *)a.gamma, (const T *)a.mean_in,
                            (const T *)a.rstd_in, partial, a.n, nchunk, 1);
-    hipLaunchKernelGGL((ln_bwd_finalize<T>), dim3(a.B), block, 0, st, partial, sample_means, a.n,
-                       nchunk);
 #define GRIDNET_LN_APPLY(V, ACC)                                                                   \
     hipLaunchKernelGGL((ln_bwd_apply<T, V, ACC>),                                                  \
                        dim3((unsigned)((a.n + (long)kLnThreads * V - 1) / ((long)kLnThreads * V))), \
                        block, 0, st, (const T *)a.dy, (const T *)a.x, (const T *)a.gamma,          \
-                       (const T *)a.mean_in, (const T *)a.rstd_in, sample_means, (T *)a.dx,        \
+                       (const T *)a.mean_in, (const T *)a.rstd_in, partial, nchunk, (T *)a.dx,     \
                        (T *)a.dgamma, (T *)a.dbeta, a.B, a.n)
     if (vec) {
         if (accum) GRIDNET_LN_APPLY(4, true); else GRIDNET_LN_APPLY(4, false);

@@ -146,14 +146,14 @@ class BodyRunner:
         if self.fused:
             return self._fused_forward(x0)
         stream = _n.current_stream(self.w)
-        self.h[0].copy_(x0)
+        self.x0 = x0  # read in place (and again by backward): the caller keeps it unchanged
         if self.has_backward:
             for j in range(self.outer):
-                self.step_forward(self.h[j], self.s[j], stream)
+                self.step_forward(self.h[j] if j else x0, self.s[j], stream)
                 self.norm_forward(self.s[j], self.h[j + 1], j, stream)
             return self.h[self.outer]
         for j in range(self.outer):  # forward only: ping-pong, nothing is kept
-            self.step_forward(self.h[j % 2], self.s[0], stream)
+            self.step_forward(self.h[j % 2] if j else x0, self.s[0], stream)
             self.norm_forward(self.s[0], self.h[(j + 1) % 2], 0, stream)
         return self.h[self.outer % 2]
 
@@ -179,7 +179,8 @@ class BodyRunner:
             # call and accumulated into by the later ones (parameters are shared)
             _n.check(_n.lib.gridnet_hip_backward(
                 self.dt, self.w.data_ptr(), self.b.data_ptr(), self.r.data_ptr(),
-                self.h[j].data_ptr(), self.ga.data_ptr(), self.dw.data_ptr(), self.db.data_ptr(),
+                (self.h[j] if j else self.x0).data_ptr(), self.ga.data_ptr(), self.dw.data_ptr(),
+                self.db.data_ptr(),
                 self.dr.data_ptr(), self.gb.data_ptr(), self.B, self.M, self.N, self.K, self.inner,
                 self.bs, self.eps, self.normalize, self.act, flags | _n.OVERWRITE_DX,
                 self.bw_ws.data_ptr(), self.bw_ws_bytes, stream))
