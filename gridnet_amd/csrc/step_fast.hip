@@ -24,14 +24,12 @@
 //   * the same delta rows give the weight gradients: x_i[c] * delta_i[c + off_t] is the gradient
 //     of the NEIGHBOUR's mirrored weight W[26-t, c + off_t], and this thread is the only one that
 //     ever contributes to it, so it accumulates in a register over iterations and batch elements
-//     (the x window is not re-read in the reverse sweep).  Weights whose tap reads a halo entry
-//     see a frozen x there: their gradient is x_halo * sum_i delta_i, one pass per batch element;
-//   * cells of neighbouring blocks (the window's halo) receive sum_t W[t,c'] * delta_i[c'] summed
-//     over i; W does not depend on i, so one pass per batch element over D = sum_i delta_i
-//     suffices.  It runs in gather form from a small LDS table (<= 9 (source, weight) pairs per
-//     halo entry, built once per workgroup) and is written, compacted, to a scratch buffer;
-//   * a second kernel adds each cell's <= 7 halo contributions from its neighbouring blocks to dx
-//     in a fixed order.
+//     (the x window is not re-read in the reverse sweep);
+//   * everything that crosses a block boundary -- what the cells of NEIGHBOURING blocks receive,
+//     and the gradient of a weight whose tap reads a (frozen) halo entry -- depends on the
+//     iterations only through D = sum_i delta_i.  The first kernel leaves D of every cell in a
+//     scratch tensor and a second kernel (step_bwd_cross), dealt by block face, works both out
+//     from the D and x windows with their real halo and completes dx, in a fixed order.
 // Parameter gradients leave the kernel once per workgroup: reduced across slots through LDS and,
 // when one workgroup owns the whole batch of its block, written with plain stores.  Results are
 // bitwise reproducible in that case.
