@@ -501,8 +501,12 @@ constexpr int kBwdDepth = 4;  // neighbour rows requested ahead of the arithmeti
 template <int BS, int CPT> __host__ __device__ constexpr int bwd_slot_floats(int inner) {
     return 4 * Tile<BS, CPT>::WIN + inner * Tile<BS, CPT>::TPS * 2 * CPT;
 }
-template <int BS, int CPT, int NSLOT> size_t bwd_lds_bytes(int inner) {
-    return (size_t)NSLOT * bwd_slot_floats<BS, CPT>(inner) * sizeof(float);
+// ... and at least the 27 weight planes of the block, which pass through LDS once at set-up
+template <int BS, int CPT, int NSLOT> size_t bwd_lds_bytes(int inner, bool ln = false) {
+    const size_t run = ((size_t)NSLOT * bwd_slot_floats<BS, CPT>(inner) + (ln ? 2 * Tile<BS, CPT>::WIN : 0)) *
+                       sizeof(float);
+    const size_t setup = (size_t)27 * BS * BS * BS * sizeof(float);
+    return run > setup ? run : setup;
 }
 
 // Commit R x C gradient values to base[index(r, c)] for the entries with ok(r, c).  One code path
@@ -574,27 +578,44 @@ void step_bwd_fast(
     for (int t = 0; t < 27; ++t) {
         load_cells<CPT>(weight + t * cells + pl.gc, w[t]);
 #pragma unroll
-        for (int c = 0; c < CPT; ++c) {
-            v[t][c] = in_block(t, c) ? weight[neighbour_weight(t, c)] : 0.f;
-            nw[t][c] = 0.f;
-        }
+        for (int c = 0; c < CPT; ++c) nw[t][c] = 0.f;
     }
     load_cells<CPT>(bias + pl.gc, bv);
     load_cells<CPT>(scale + pl.gc, rv);
 #pragma unroll
     for (int c = 0; c < CPT; ++c) db[c] = dr[c] = 0.f;
     float gam[CPT], dgam[CPT], dbet[CPT];
-    typename Fetch<TL>::Buf pre;
     if (LN) {
         load_cells<CPT>(ln.gamma + pl.gc, gam);
 #pragma unroll
         for (int c = 0; c < CPT; ++c) dgam[c] = dbet[c] = 0.f;
-        if (ln_in && pl.slot == 0) {  // gamma and beta of the window, once per workgroup
-            fx.fetch(ln.gamma, pre);
-            fx.template commit<1>(gwin, pre);
-            fx.fetch(ln.beta, pre);
-            fx.template commit<1>(bwin, pre);
+    }
+    {   // The mirrored neighbour weights are other threads' w: they are exchanged through LDS
+        // (the windows are not in use yet) instead of read from global memory a second time --
+        // every workgroup of the grid does this at the same moment, and twice the weight tensor
+        // was what the set-up phase waited for.
+        constexpr int NC = BS * BS * BS;
+        float *wl = lds;  // [27][NC], by block-local cell (i, j, k)
+        const int lin = (pl.i * BS + pl.j) * BS + pl.kt * CPT;
+        if (pl.slot == 0) {
+#pragma unroll
+            for (int t = 0; t < 27; ++t) store_cells<CPT>(wl + t * NC + lin, w[t]);
         }
+        lds_barrier();
+#pragma unroll
+        for (int t = 0; t < 27; ++t)
+#pragma unroll
+            for (int c = 0; c < CPT; ++c)
+                v[t][c] = in_block(t, c) ? wl[(26 - t) * NC + lin + c + ((t / 9 - 1) * BS + ((t / 3) % 3 - 1)) * BS + (t % 3 - 1)]
+                                         : 0.f;
+        lds_barrier();  // the windows reuse this memory
+    }
+    typename Fetch<TL>::Buf pre;
+    if (ln_in && pl.slot == 0) {  // gamma and beta of the window, once per workgroup
+        fx.fetch(ln.gamma, pre);
+        fx.template commit<1>(gwin, pre);
+        fx.fetch(ln.beta, pre);
+        fx.template commit<1>(bwin, pre);
     }
 
     // delta windows: the halo stays zero for the whole kernel
@@ -1133,7 +1154,7 @@ template <int BS, int CPT, int NSLOT, int ACT, bool LN>
 int launch_bwd_ln(const StepArgs &a, hipStream_t st) {
     using TL = Tile<BS, CPT>;
     const long cells = (long)a.M * a.N * a.K;
-    const size_t lds = bwd_lds_bytes<BS, CPT, NSLOT>(a.inner) + (LN ? 2 * TL::WIN * sizeof(float) : 0);
+    const size_t lds = bwd_lds_bytes<BS, CPT, NSLOT>(a.inner, LN);
     auto kern = step_bwd_fast<BS, CPT, NSLOT, ACT, LN>;
     static bool big_lds_enabled = false;            // per instantiation
     static int per_cu_cache[kMaxBackwardIters + 1];  // per instantiation, by inner iterations
@@ -1232,9 +1253,9 @@ bool step_fast_supports(const StepArgs &a, bool backward) {
     if (a.dtype != GRIDNET_F32 || a.normalize) return false;
     if (a.block_size != 4 && a.block_size != 8) return false;
     if (backward) {
-        size_t lds = a.block_size == 8 ? bwd_lds_bytes<8, kBwdCpt8, kBwdSlots8>(a.inner)
-                                       : bwd_lds_bytes<4, kBwdCpt4, kBwdSlots4>(a.inner);
-        if (a.ln.gamma) lds += 2 * (a.block_size == 8 ? Tile<8, 1>::WIN : Tile<4, 1>::WIN) * sizeof(float);
+        const bool ln = a.ln.gamma != nullptr;
+        const size_t lds = a.block_size == 8 ? bwd_lds_bytes<8, kBwdCpt8, kBwdSlots8>(a.inner, ln)
+                                             : bwd_lds_bytes<4, kBwdCpt4, kBwdSlots4>(a.inner, ln);
         if (lds > kMaxLds) return false;
     }
     return true;
