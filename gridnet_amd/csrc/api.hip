@@ -64,7 +64,7 @@ using namespace gridnet;
 
 extern "C" {
 
-int gridnet_hip_version(void) { return 1; }
+int gridnet_hip_version(void) { return 2; }  // 2: fused body entry points
 
 const char *gridnet_hip_last_error(void) { return error_buffer(); }
 
