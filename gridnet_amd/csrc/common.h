@@ -93,6 +93,58 @@ template <typename T> __device__ __forceinline__ T block_sum(T v, T *scratch, in
     return total;
 }
 
+// ---- device: gathering what a block's cells send to the window around it -----------------
+// In the backward of a block-local update every cell c sends weight[t][c] * delta[c] to window
+// entry c + offset(t), t = 9a+3b+c' <-> offset (a-1, b-1, c'-1).  Scattering that with LDS float
+// atomics is slow (ds_add_f32: the fp32 kernels took 3x as long as with this gather), so the
+// one-thread-per-cell fp32 kernels publish their 27 products in a table prod[27][bs^3] and every
+// window entry e sums the ones aimed at it: tap t from cell e - offset(t), where that cell exists.
+// ds_add_f64 keeps up, and an fp64 table would leave room for one workgroup per CU only (measured
+// 1.7x slower than the scatter), so fp64 keeps the atomics.
+template <typename T> constexpr bool kGatherTaps = sizeof(T) == 4;
+
+template <int BS> struct TapGather {
+    static constexpr int S = BS + 2, W = S * S * S, NT = BS * BS * BS;
+    static constexpr int kEntries = (W + NT - 1) / NT;  // window entries per thread
+    static constexpr int kLinBias = (BS + 1) * BS * BS;  // halo entries have cell indices < 0
+
+    // Descriptor of window entry idx: per axis, which of the three offsets lead back into the
+    // block (bits 0-2, 3-5, 6-8), and above them the biased linear cell index of the entry.
+    static __device__ __forceinline__ unsigned describe(int idx) {
+        const int wk = idx % S, wj = (idx / S) % S, wi = idx / (S * S);
+        unsigned bits = 0;
+#pragma unroll
+        for (int o = 0; o < 3; ++o) {
+            const int si = wi - (o - 1), sj = wj - (o - 1), sk = wk - (o - 1);  // source, window coords
+            if (si >= 1 && si <= BS) bits |= 1u << o;
+            if (sj >= 1 && sj <= BS) bits |= 8u << o;
+            if (sk >= 1 && sk <= BS) bits |= 64u << o;
+        }
+        if (idx >= W) bits = 0;
+        const int lin = ((wi - 1) * BS + (wj - 1)) * BS + (wk - 1);
+        return bits | ((unsigned)(lin + kLinBias) << 9);
+    }
+
+    template <typename T>
+    static __device__ __forceinline__ T collect(const T *prod, unsigned desc) {
+        const int lin = (int)(desc >> 9) - kLinBias;
+        T acc = T(0);
+#pragma unroll
+        for (int a = 0; a < 3; ++a)
+#pragma unroll
+            for (int b = 0; b < 3; ++b)
+#pragma unroll
+                for (int c = 0; c < 3; ++c) {
+                    const unsigned bit = (1u << a) | (8u << b) | (64u << c);
+                    const bool ok = (desc & bit) == bit;
+                    const int src = lin - (((a - 1) * BS + (b - 1)) * BS + (c - 1));
+                    const T p = prod[(a * 9 + b * 3 + c) * NT + (ok ? src : 0)];
+                    acc += ok ? p : T(0);
+                }
+        return acc;
+    }
+};
+
 // Workgroup id -> (spatial block, batch chunk).  Workgroup ids are dealt to the 8 XCDs
 // round-robin and every XCD has its own L2, so XCD x is given a CONTIGUOUS range of spatial
 // blocks (raster order: neighbours along K, then N): neighbouring blocks share halo cells and

@@ -100,9 +100,15 @@ __global__ __launch_bounds__(BS *BS *BS) void gated_bwd(
     using G = GGeo<BS>;
     __shared__ T win[G::W];   // window state x_i
     __shared__ T gwin[G::W];  // dL/d(window); the owned entry is rewritten every iteration
+    // fp32: the cells' 27 products, gathered by the window entries instead of LDS float atomics
+    using Gather = TapGather<BS>;
+    __shared__ T prod[kGatherTaps<T> ? 27 * G::NT : 1];
     const int tid = threadIdx.x;
     int blk, chunk;
     if (!split_block_id(blockIdx.x, nblk, nchunk, blk, chunk)) return;
+    unsigned entry[Gather::kEntries];  // the window entries this thread gathers for
+#pragma unroll
+    for (int e = 0; e < Gather::kEntries; ++e) entry[e] = Gather::describe(tid + e * G::NT);
     const int kb = K / BS, nb = N / BS;
     const int p0 = (blk / (kb * nb)) * BS, q0 = ((blk / kb) % nb) * BS, r0 = (blk % kb) * BS;
     const int ci = tid / (BS * BS), cj = (tid / BS) % BS, ck = tid % BS;
@@ -164,9 +170,20 @@ __global__ __launch_bounds__(BS *BS *BS) void gated_bwd(
                         const T v = win[o];
                         dwa[t] += v * dpre;
                         dwg[t] += v * dgpre;
-                        atomicAdd(&gwin[o], wa[t] * dpre + wg[t] * dgpre);
+                        const T sent = wa[t] * dpre + wg[t] * dgpre;
+                        if (kGatherTaps<T>) prod[t * G::NT + tid] = sent;
+                        else atomicAdd(&gwin[o], sent);
                     }
             __syncthreads();
+            if (kGatherTaps<T>) {
+#pragma unroll
+                for (int e = 0; e < Gather::kEntries; ++e) {
+                    const int idx = tid + e * G::NT;
+                    const T acc = Gather::collect(prod, entry[e]);
+                    if (idx < G::W) gwin[idx] += acc;
+                }
+                __syncthreads();
+            }
             g = gwin[centre];
         }
         if (inner == 0) gwin[centre] = g;

@@ -117,6 +117,15 @@ __global__ __launch_bounds__(BS *BS *BS) void step_fwd_generic(
     }
 }
 
+// LDS of the backward kernel: three windows, the table of per-tap products and the reduction
+// scratch.  Above 64 KB for fp64 at block size 8, hence dynamic.
+extern __shared__ __align__(16) unsigned char generic_lds[];
+
+template <typename T, int BS> constexpr size_t bwd_generic_lds() {
+    return (3 * Geo<BS>::W + (kGatherTaps<T> ? 27 * Geo<BS>::NT : 0) + 8 + 3 * kMaxBackwardIters) *
+           sizeof(T);
+}
+
 template <typename T, int BS, int ACT, bool NORM>
 __global__ __launch_bounds__(BS *BS *BS) void step_bwd_generic(
     const T *__restrict__ weight, const T *__restrict__ bias, const T *__restrict__ scale,
@@ -124,10 +133,12 @@ __global__ __launch_bounds__(BS *BS *BS) void step_bwd_generic(
     T *__restrict__ dbias, T *__restrict__ dscale, T *__restrict__ dx, int B, int M, int N, int K,
     int inner, T eps, int nblk, int nchunk, int chunk_len, int param_mode) {
     using G = Geo<BS>;
-    __shared__ T win[G::W];   // state v_i of the window
-    __shared__ T gwin[G::W];  // dL/d(window), carried through the iterations
-    __shared__ T dz[G::W];    // dL/d(stencil input) of the current iteration
-    __shared__ T red[8];
+    T *win = reinterpret_cast<T *>(generic_lds);  // state v_i of the window
+    T *gwin = win + G::W;                         // dL/d(window), carried through the iterations
+    T *dz = gwin + G::W;                          // dL/d(stencil input) of the current iteration
+    T *prod = dz + G::W;                          // [27][cells]: weight * delta of every cell
+    T *red = prod + (kGatherTaps<T> ? 27 * G::NT : 0);
+    T *stat = red + 8;  // (mean, std, 1/(std+eps)) of the window before each inner iteration
 
     const int tid = threadIdx.x;
     int blk, chunk;
@@ -150,6 +161,11 @@ __global__ __launch_bounds__(BS *BS *BS) void step_bwd_generic(
     T db = T(0), dr = T(0);
     T hist[kMaxBackwardIters];  // this cell's value before each inner iteration
 
+    using Gather = TapGather<BS>;
+    unsigned entry[Gather::kEntries];  // the window entries this thread gathers for
+#pragma unroll
+    for (int e = 0; e < Gather::kEntries; ++e) entry[e] = Gather::describe(tid + e * G::NT);
+
     const int s_end = min(B, (chunk + 1) * chunk_len);
     for (int s = chunk * chunk_len; s < s_end; ++s) {
         load_window<T, BS>(win, x + s * cells, p0, q0, r0, M, N, K, tid);
@@ -162,7 +178,14 @@ __global__ __launch_bounds__(BS *BS *BS) void step_bwd_generic(
         for (int it = 0; it < inner; ++it) {
             hist[it] = cur;
             T mean = T(0), sd = T(0), inv = T(1);
-            if (NORM) window_stats<T, BS>(win, red, tid, eps, mean, sd, inv);
+            if (NORM) {
+                window_stats<T, BS>(win, red, tid, eps, mean, sd, inv);
+                if (tid == 0) {
+                    stat[3 * it] = mean;
+                    stat[3 * it + 1] = sd;
+                    stat[3 * it + 2] = inv;
+                }
+            }
             const T u = pre_activation<T, BS, NORM>(win, w, bv, base, mean, inv);
             cur += rv * Act<ACT, T>::f(u);
             __syncthreads();
@@ -172,10 +195,15 @@ __global__ __launch_bounds__(BS *BS *BS) void step_bwd_generic(
 
         for (int it = inner - 1; it >= 0; --it) {
             win[centre] = hist[it];  // window back to state v_it (the halo never changed)
-            for (int idx = tid; idx < G::W; idx += G::NT) dz[idx] = T(0);
+            if (!kGatherTaps<T>)
+                for (int idx = tid; idx < G::W; idx += G::NT) dz[idx] = T(0);
             __syncthreads();
             T mean = T(0), sd = T(0), inv = T(1);
-            if (NORM) window_stats<T, BS>(win, red, tid, eps, mean, sd, inv);
+            if (NORM) {  // as the recompute found them: the window is back in that state
+                mean = stat[3 * it];
+                sd = stat[3 * it + 1];
+                inv = stat[3 * it + 2];
+            }
             const T u = pre_activation<T, BS, NORM>(win, w, bv, base, mean, inv);
             T f, d;
             Act<ACT, T>::fd(u, f, d);
@@ -189,13 +217,21 @@ __global__ __launch_bounds__(BS *BS *BS) void step_bwd_generic(
                 for (int b = 0; b < 3; ++b)
 #pragma unroll
                     for (int c = 0; c < 3; ++c) {
-                        const int o = base + (a * G::S + b) * G::S + c;
-                        T v = win[o];
+                        const int t = a * 9 + b * 3 + c;
+                        T v = win[base + (a * G::S + b) * G::S + c];
                         if (NORM) v = (v - mean) * inv;
-                        dw[a * 9 + b * 3 + c] += v * delta;
-                        atomicAdd(&dz[o], w[a * 9 + b * 3 + c] * delta);
+                        dw[t] += v * delta;
+                        if (kGatherTaps<T>) prod[t * G::NT + tid] = w[t] * delta;
+                        else atomicAdd(&dz[base + (a * G::S + b) * G::S + c], w[t] * delta);
                     }
             __syncthreads();
+#pragma unroll
+            for (int e = 0; e < (kGatherTaps<T> ? Gather::kEntries : 0); ++e) {
+                const int idx = tid + e * G::NT;
+                const T acc = Gather::collect(prod, entry[e]);
+                if (idx < G::W) dz[idx] = acc;
+            }
+            if (kGatherTaps<T>) __syncthreads();
             if (NORM) {
                 // z = (v - mean) * inv over the whole window: push dz back through it
                 T sdz = T(0), sproj = T(0);
@@ -265,19 +301,34 @@ int launch_fwd_norm(const StepArgs &a, int nblk, int nchunk, int chunk_len, hipS
     return check_launch("step_fwd_generic");
 }
 
+template <typename T, int BS, int ACT, bool NORM>
+int launch_bwd_kernel(const StepArgs &a, int nblk, int nchunk, int chunk_len, int param_mode,
+                      hipStream_t st) {
+    dim3 grid(padded_grid(nblk, nchunk)), block(Geo<BS>::NT);
+    auto kern = step_bwd_generic<T, BS, ACT, NORM>;
+    constexpr size_t lds = bwd_generic_lds<T, BS>();
+    static bool big_lds_enabled = false;  // per instantiation
+    if (lds > 64 * 1024 && !big_lds_enabled) {
+        hipError_t e = hipFuncSetAttribute((const void *)kern,
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess)
+            return fail(GRIDNET_ERR_LAUNCH, "cannot enable %zu bytes of LDS: %s", lds,
+                        hipGetErrorString(e));
+        big_lds_enabled = true;
+    }
+    hipLaunchKernelGGL(kern, grid, block, lds, st, (const T *)a.weight, (const T *)a.bias,
+                       (const T *)a.scale, (const T *)a.x, (const T *)a.dy, (T *)a.dweight,
+                       (T *)a.dbias, (T *)a.dscale, (T *)a.dx, a.B, a.M, a.N, a.K, a.inner,
+                       (T)a.eps, nblk, nchunk, chunk_len, param_mode);
+    return check_launch("step_bwd_generic");
+}
+
 template <typename T, int BS, int ACT>
 int launch_bwd_norm(const StepArgs &a, int nblk, int nchunk, int chunk_len, int param_mode,
                     hipStream_t st) {
-    dim3 grid(padded_grid(nblk, nchunk)), block(Geo<BS>::NT);
-    auto args = [&](auto kern) {
-        hipLaunchKernelGGL(kern, grid, block, 0, st, (const T *)a.weight, (const T *)a.bias,
-                           (const T *)a.scale, (const T *)a.x, (const T *)a.dy, (T *)a.dweight,
-                           (T *)a.dbias, (T *)a.dscale, (T *)a.dx, a.B, a.M, a.N, a.K, a.inner,
-                           (T)a.eps, nblk, nchunk, chunk_len, param_mode);
-    };
-    if (a.normalize) args(step_bwd_generic<T, BS, ACT, true>);
-    else args(step_bwd_generic<T, BS, ACT, false>);
-    return check_launch("step_bwd_generic");
+    if (a.normalize)
+        return launch_bwd_kernel<T, BS, ACT, true>(a, nblk, nchunk, chunk_len, param_mode, st);
+    return launch_bwd_kernel<T, BS, ACT, false>(a, nblk, nchunk, chunk_len, param_mode, st);
 }
 
 template <typename T, int BS, bool BWD>
