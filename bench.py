@@ -47,6 +47,32 @@ def gpu_run(wl, steps, warmup, fused):
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
 
+    # The same step as one captured HIP graph, replayed: what is left when the host side (Python,
+    # ctypes, launch calls) is taken out.  Reported beside the eager figure, which stays the headline.
+    graph_s = None
+    try:
+        side = torch.cuda.Stream(device=dev)
+        side.wait_stream(torch.cuda.current_stream(dev))
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            one_step()  # this stream's first use, outside the capture
+            side.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                one_step()
+            for _ in range(max(1, warmup)):
+                graph.replay()
+            side.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                graph.replay()
+            side.synchronize()
+            graph_s = (time.perf_counter() - t0) / steps
+        torch.cuda.current_stream(dev).wait_stream(side)
+        del graph
+    except RuntimeError as exc:  # reported, not fatal: the headline does not depend on it
+        print(f"bench.py: HIP graph replay skipped: {exc}", file=sys.stderr, flush=True)
+    torch.cuda.synchronize()
+
     # per-entry-point device time: events recorded on the stream the kernels are launched on
     # (torch's current stream is the one handed to the C ABI), in a separate instrumented pass
     spans = {}
@@ -67,7 +93,7 @@ def gpu_run(wl, steps, warmup, fused):
         assert p0 == 0 and p1 == 1
         spans.setdefault(name, []).append(e0.elapsed_time(e1) * 1e-3)
     kernel_s = {k: sum(v) / len(v) for k, v in spans.items()}
-    return wall, kernel_s
+    return wall, graph_s, kernel_s
 
 
 def cpu_baseline(wl, budget_s=25.0):
@@ -135,7 +161,7 @@ def main():
 
     wl = WORKLOADS[args.workload]
     fused = args.path == "fused" and not wl.normalize and wl.inner >= 1
-    wall, kernel_s = gpu_run(wl, args.steps, args.warmup, fused)
+    wall, graph_s, kernel_s = gpu_run(wl, args.steps, args.warmup, fused)
     bytes_ = wl.algorithmic_bytes()
     if fused:  # a fused entry point does the work of the step AND of the LayerNorm beside it
         bytes_["step_fwd"] += bytes_["ln_fwd"]
@@ -167,6 +193,9 @@ def main():
         "config": {"workload": wl.name, "activation": wl.activation, "normalize": wl.normalize,
                    "pass": "fwd+bwd" if wl.backward else "fwd",
                    "path": "fused step+LayerNorm entry points" if fused else "step and LayerNorm calls"},
+        "timing": {"headline": "eager wall clock over the timed steps, synchronised on both sides",
+                   "eager_ms_per_step": wall * 1e3,
+                   "hip_graph_replay_ms_per_step": None if graph_s is None else graph_s * 1e3},
         "hbm_roofline_frac_whole_step": bytes_["total"] / wall / (HBM_PEAK_GBS * 1e9),
         "entry_point_ms": {k: v * 1e3 for k, v in kernel_s.items()},
         "roofline": {
