@@ -1148,7 +1148,7 @@ constexpr size_t kMaxLds = 160 * 1024;
 
 // the cross-block kernel's own shapes (it shares the main kernel's blocks and batch chunks)
 constexpr int kCrossSlots8 = 1, kCrossElems8 = 2;  // bs=8: 384 threads, one wave per face
-constexpr int kCrossSlots4 = 4, kCrossElems4 = 2;  // bs=4: four slots of 96 threads
+constexpr int kCrossSlots4 = 2, kCrossElems4 = 2;  // bs=4: two slots of 96 threads
 
 template <int BS, int CPT, int NSLOT, int ACT, bool LN>
 int launch_bwd_ln(const StepArgs &a, hipStream_t st) {
@@ -1220,7 +1220,7 @@ template <int BS, int CPT, int NSLOT, int ACT> int launch_bwd(const StepArgs &a,
 constexpr int kFwdCpt8 = 4, kFwdSlots8 = 1;   // bs=8 forward: 128 threads, 4 cells each
 constexpr int kBwdCpt8 = 2, kBwdSlots8 = 1;   // bs=8 backward: 256 threads, 2 cells each
 constexpr int kFwdCpt4 = 2, kFwdSlots4 = 4;   // bs=4: 32-thread slots, 4 per workgroup
-constexpr int kBwdCpt4 = 1, kBwdSlots4 = 2;   // bs=4 backward: one wave per slot, one cell per thread
+constexpr int kBwdCpt4 = 2, kBwdSlots4 = 2;   // bs=4 backward: two 32-thread slots, 2 cells per thread
 
 template <bool BWD, int ACT> int dispatch_bs(const StepArgs &a, hipStream_t st) {
     if (a.block_size == 8) {
