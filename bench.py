@@ -20,7 +20,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor peak
 
 
-def gpu_run(wl, steps, warmup, fused):
+def gpu_run(wl, steps, warmup, fused, graph_replay=True):
     import torch
 
     from gridnet_amd.configs import make_inputs
@@ -51,6 +51,8 @@ def gpu_run(wl, steps, warmup, fused):
     # ctypes, launch calls) is taken out.  Reported beside the eager figure, which stays the headline.
     graph_s = None
     try:
+        if not graph_replay:
+            raise RuntimeError("switched off (--no-graph)")
         side = torch.cuda.Stream(device=dev)
         side.wait_stream(torch.cuda.current_stream(dev))
         graph = torch.cuda.CUDAGraph()
@@ -153,6 +155,8 @@ def main():
                          "(the faster of the two on MI355X as measured); fused: the entry points "
                          "with the LayerNorm folded into the step kernels")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="skip the HIP graph replay (for runs under a counter-collecting profiler)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (no collectives, no sharding); "
@@ -161,7 +165,7 @@ def main():
 
     wl = WORKLOADS[args.workload]
     fused = args.path == "fused" and not wl.normalize and wl.inner >= 1
-    wall, graph_s, kernel_s = gpu_run(wl, args.steps, args.warmup, fused)
+    wall, graph_s, kernel_s = gpu_run(wl, args.steps, args.warmup, fused, not args.no_graph)
     bytes_ = wl.algorithmic_bytes()
     if fused:  # a fused entry point does the work of the step AND of the LayerNorm beside it
         bytes_["step_fwd"] += bytes_["ln_fwd"]
