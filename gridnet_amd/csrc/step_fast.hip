@@ -493,6 +493,167 @@ void step_fwd_fast(
     if (done_s >= 0) store_cells<CPT>(y + done_s * cells + pl.gc, done);
 }
 
+// ---- forward, 8^3 blocks: the split window ------------------------------------------------
+// The LDS pipeline limits step_fwd_fast at this block size as much as the vector ALU does: a
+// thread's 6-float row is a 128-bit plus a 64-bit read whose lanes collide on banks, and the
+// results go back as unaligned 32-bit writes that use a quarter of the banks.  This kernel keeps
+// the window in two parts instead:
+//   * centre: the 8 block columns of every window row as 8 floats, the second four REVERSED
+//     (columns 0 1 2 3 7 6 5 4).  A thread owns four cells of a row, holds them in the order
+//     they are stored, and reads or writes them as one aligned, conflict-free 128-bit access;
+//   * side: the two halo columns of every row, dense, one 32-bit read per row.
+// The sixth value of a row, the cell next to the thread's four on the inner side, is the last
+// register of the lane that owns the other half of the row (lane ^ 1): one DPP operand, no LDS.
+// With the second half reversed both lanes of a pair see the same picture -- [side entry, own
+// four cells outward-in, partner's cell] -- so the code is uniform; the lanes of the second
+// half hold their weights mirrored along K to match.
+struct SplitWin {
+    static constexpr int S = 10, RS = 8, PS = S * RS;  // centre rows and planes (floats)
+    static constexpr int CEN = S * PS;
+    static constexpr int SP = 12, SS = S * SP;         // side rows of 10 at stride 12, per side
+    static constexpr int COPY = CEN + 2 * SS;          // floats per window copy
+};
+
+// value of `v` in the lane that owns the other half of the row (lanes 2m and 2m+1 swap)
+__device__ __forceinline__ float partner_lane(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true));
+}
+
+template <int ACT>
+__global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(3)))
+void step_fwd_split(
+    const float *__restrict__ weight, const float *__restrict__ bias,
+    const float *__restrict__ scale, const float *__restrict__ x, float *__restrict__ y, int B, int M,
+    int N, int K, int inner, int nblk, int nchunk, int chunk_len) {
+    using TL = Tile<8, 4>;
+    using SW = SplitWin;
+    using FX = Fetch<TL>;
+    __shared__ __attribute__((aligned(16))) float lds[2 * SW::COPY];
+
+    int blk, chunk;
+    if (!split_block_id(blockIdx.x, nblk, nchunk, blk, chunk)) return;  // grid padding
+    const Place<TL, 4, 1> pl(threadIdx.x, blk, N, K);
+    const FX fx(pl.lane, pl.p0, pl.q0, pl.r0, M, N, K);
+    const long cells = (long)M * N * K;
+    const bool second = pl.kt != 0;  // this thread holds columns 7 6 5 4, in that order
+
+    // where this thread's half rows go: the four cells into the centre part, the end entry
+    // into the side part of its half
+    int cen_at[FX::RPT], side_at[FX::RPT];
+#pragma unroll
+    for (int e = 0; e < FX::RPT; ++e) {
+        const int id = pl.lane + e * TL::TPS;
+        const int half = id & 1, row = id >> 1;
+        const int wj = row % SW::S, wi = row / SW::S;
+        cen_at[e] = wi * SW::PS + wj * SW::RS + half * 4;
+        side_at[e] = SW::CEN + half * SW::SS + wi * SW::SP + wj;
+    }
+    // tap (a, b) of this thread's rows: centre vector and side entry
+    const int cen00 = pl.i * SW::PS + pl.j * SW::RS + pl.kt * 4;
+    const int side00 = SW::CEN + pl.kt * SW::SS + pl.i * SW::SP + pl.j;
+    const int own = cen00 + SW::PS + SW::RS;
+
+    // Parameters in register order.  First half: w[t][r] is tap t of column r.  Second half:
+    // register r is column 7-r and a step of one register is a step of -1 along K, so the tap
+    // with K-offset cc sits at register offset 2-cc.
+    float w[27][4], bv[4], rv[4];
+#pragma unroll
+    for (int ab = 0; ab < 9; ++ab) {
+        float wt[3][4];
+#pragma unroll
+        for (int cc = 0; cc < 3; ++cc) load_cells<4>(weight + (ab * 3 + cc) * cells + pl.gc, wt[cc]);
+#pragma unroll
+        for (int cc = 0; cc < 3; ++cc)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) w[ab * 3 + cc][r] = second ? wt[2 - cc][3 - r] : wt[cc][r];
+    }
+    {
+        float bt[4], rt[4];
+        load_cells<4>(bias + pl.gc, bt);
+        load_cells<4>(scale + pl.gc, rt);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            bv[r] = second ? bt[3 - r] : bt[r];
+            rv[r] = second ? rt[3 - r] : rt[r];
+        }
+    }
+    wait_global_loads();
+
+    auto commit = [&](const typename FX::Buf &v) {
+#pragma unroll
+        for (int e = 0; e < FX::RPT; ++e)
+            if (fx.loff[e] >= 0) {
+                const float end = (fx.ok[e] && fx.edge_ok[e]) ? v[e][4] : 0.f;
+                float c[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) c[r] = fx.ok[e] ? (fx.hi[e] ? v[e][3 - r] : v[e][r]) : 0.f;
+#pragma unroll
+                for (int copy = 0; copy < 2; ++copy) {
+                    *reinterpret_cast<float4 *>(lds + copy * SW::COPY + cen_at[e]) =
+                        make_float4(c[0], c[1], c[2], c[3]);
+                    lds[copy * SW::COPY + side_at[e]] = end;
+                }
+            }
+    };
+    auto store_result = [&](int s, const float (&cur)[4]) {
+        float out[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) out[c] = second ? cur[3 - c] : cur[c];
+        store_cells<4>(y + s * cells + pl.gc, out);
+    };
+
+    const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
+    typename FX::Buf pre;
+    if (s0 < s1) fx.fetch(x + s0 * cells, pre);
+    // The result of an element is stored one element late, after the next window has been
+    // committed (see step_fwd_fast).
+    float done[4];
+    int done_s = -1;
+    for (int s = s0; s < s1; ++s) {
+        commit(pre);
+        lds_barrier();
+        if (done_s >= 0) store_result(done_s, done);
+        if (s + 1 < s1) fx.fetch(x + (s + 1) * cells, pre);  // next element, in flight
+        float cur[4];
+        {
+            const float4 q = *reinterpret_cast<const float4 *>(lds + own);
+            cur[0] = q.x; cur[1] = q.y; cur[2] = q.z; cur[3] = q.w;
+        }
+        for (int it = 0; it < inner; ++it) {
+            const float *from = lds + (it & 1) * SW::COPY;
+            float u[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) u[r] = bv[r];
+#pragma unroll
+            for (int a = 0; a < 3; ++a)
+#pragma unroll
+                for (int b = 0; b < 3; ++b) {
+                    const float4 q =
+                        *reinterpret_cast<const float4 *>(from + cen00 + a * SW::PS + b * SW::RS);
+                    float v[6];
+                    v[0] = from[side00 + a * SW::SP + b];
+                    v[1] = q.x; v[2] = q.y; v[3] = q.z; v[4] = q.w;
+                    v[5] = partner_lane(q.w);
+#pragma unroll
+                    for (int cc = 0; cc < 3; ++cc)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            u[r] = fmaf(w[a * 9 + b * 3 + cc][r], v[r + cc], u[r]);
+                }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) cur[r] = fmaf(rv[r], Act<ACT, float>::f(u[r]), cur[r]);
+            *reinterpret_cast<float4 *>(lds + ((it + 1) & 1) * SW::COPY + own) =
+                make_float4(cur[0], cur[1], cur[2], cur[3]);
+            lds_barrier();
+        }
+        done_s = s;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) done[r] = cur[r];
+        if (inner == 0) lds_barrier();  // `cur` was read from the window that is rewritten next
+    }
+    if (done_s >= 0) store_result(done_s, done);
+}
+
 // ---- backward ------------------------------------------------------------------------------
 constexpr int kBwdDepth = 4;  // neighbour rows requested ahead of the arithmetic
 
@@ -1139,8 +1300,24 @@ template <int BS, int CPT, int NSLOT, int ACT, bool LN> int launch_fwd_ln(const 
                        p.chunk_len, a.ln);
     return check_launch("step_fwd_fast");
 }
+template <int ACT> int launch_fwd_split(const StepArgs &a, hipStream_t st) {
+    auto kern = step_fwd_split<ACT>;
+    static int per_cu = 0;
+    if (per_cu == 0) {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, 128, 0) != hipSuccess || n < 1) n = 1;
+        per_cu = n;
+    }
+    const Plan p = make_plan(a, 1, per_cu * device_cus(), false);
+    hipLaunchKernelGGL(kern, dim3(padded_grid(p.nblk, p.nchunk)), dim3(128), 0, st,
+                       (const float *)a.weight, (const float *)a.bias, (const float *)a.scale,
+                       (const float *)a.x, (float *)a.y, a.B, a.M, a.N, a.K, a.inner, p.nblk, p.nchunk,
+                       p.chunk_len);
+    return check_launch("step_fwd_split");
+}
 template <int BS, int CPT, int NSLOT, int ACT> int launch_fwd(const StepArgs &a, hipStream_t st) {
     if (a.ln.gamma) return launch_fwd_ln<BS, CPT, NSLOT, ACT, true>(a, st);
+    if (BS == 8) return launch_fwd_split<ACT>(a, st);
     return launch_fwd_ln<BS, CPT, NSLOT, ACT, false>(a, st);
 }
 
