@@ -717,10 +717,14 @@ void step_bwd_fast(
     float *win = lds + pl.slot * slot_floats;
     float *dwin = win + 2 * TL::WIN;
     float *hist = dwin + 2 * TL::WIN + pl.lane * CPT;  // + it*TPS*2*CPT (x_i), + TPS*CPT more (u_i)
+    // The x window copy that would receive x_inner (never needed) gets zeros in the block's
+    // cells instead: the x window's halo alone, for the weights of the taps that read it.
+    const float *xhalo = win + (inner & 1) * TL::WIN;
     float *gwin = lds + NSLOT * slot_floats, *bwin = gwin + TL::WIN;  // LN: gamma, beta windows
     const long cells = (long)M * N * K;
 
-    // nw[t][c] belongs to the weight of the neighbour at c + off_t, where that lies in this block
+    // nw[t][c] belongs to the weight of the neighbour at c + off_t where that lies in this block,
+    // and to this cell's own weight of tap t where it does not (see below)
     auto in_block = [&](int t, int c) {
         const int ni = pl.i + t / 9 - 1, nj = pl.j + (t / 3) % 3 - 1, nk = pl.kt * CPT + c + t % 3 - 1;
         return ni >= 0 && ni < BS && nj >= 0 && nj < BS && nk >= 0 && nk < BS;
@@ -728,12 +732,20 @@ void step_bwd_fast(
     auto neighbour_weight = [&](int t, int c) {
         return (26 - t) * cells + pl.gc + c + ((t / 9 - 1) * N + ((t / 3) % 3 - 1)) * K + (t % 3 - 1);
     };
+    auto owner_of = [&](int t, int c) {
+        return in_block(t, c) ? neighbour_weight(t, c) : t * cells + pl.gc + c;
+    };
+    auto always = [](int, int) { return true; };
 
     // ---- once per workgroup: parameters and mirrored neighbour weights ----
     // w : this cell's weights (forward recompute)
     // v : V[t][c] = W[26-t, c + off_t], what the neighbour at c + off_t multiplies cell c by
     // nw: gradient of that same neighbour weight; it is the product of this cell's x and the
-    //     neighbour's delta summed over iterations and batch, so this thread owns it completely
+    //     neighbour's delta summed over iterations and batch, so this thread owns it completely.
+    //     Where the neighbour lies in ANOTHER block the slot would stay empty (the delta halo is
+    //     zero); it holds the gradient of this cell's own weight of tap t instead: that tap reads
+    //     a halo entry, frozen over the iterations, so its gradient is x_halo[c + off_t] * D[c]
+    //     with D = sum_i delta_i, added once per element from a window that holds the halo alone.
     float w[27][CPT], v[27][CPT], nw[27][CPT], bv[CPT], rv[CPT], db[CPT], dr[CPT];
 #pragma unroll
     for (int t = 0; t < 27; ++t) {
@@ -789,8 +801,7 @@ void step_bwd_fast(
 #pragma unroll
         for (int t = 0; t < 27; ++t)
 #pragma unroll
-            for (int c = 0; c < CPT; ++c)
-                if (in_block(t, c)) nw[t][c] = dweight[neighbour_weight(t, c)];
+            for (int c = 0; c < CPT; ++c) nw[t][c] = dweight[owner_of(t, c)];
 #pragma unroll
         for (int c = 0; c < CPT; ++c) {
             db[c] = dbias[pl.gc + c];
@@ -879,12 +890,15 @@ void step_bwd_fast(
                 float *h = hist + it * (TL::TPS * 2 * CPT);
                 store_cells<CPT>(h, cur);
                 store_cells<CPT>(h + TL::TPS * CPT, u);
-                if (it + 1 < inner) {  // x_inner itself is never needed
+                if (it + 1 < inner) {
 #pragma unroll
                     for (int c = 0; c < CPT; ++c) {
                         cur[c] = fmaf(rv[c], Act<ACT, float>::f(u[c]), cur[c]);
                         win[((it + 1) & 1) * TL::WIN + pl.own + c] = cur[c];
                     }
+                } else {  // x_inner itself is never needed: that copy becomes the halo window
+#pragma unroll
+                    for (int c = 0; c < CPT; ++c) win[((it + 1) & 1) * TL::WIN + pl.own + c] = 0.f;
                 }
             }
             if (it + 1 < inner) lds_barrier();
@@ -910,6 +924,21 @@ void step_bwd_fast(
                     dsum[c] += delta;
                     dwin[(it & 1) * TL::WIN + pl.own + c] = delta;
                 }
+            }
+            if (it == 0) {
+                // D is complete: the weights of the taps that read the halo.  Before this
+                // iteration's barrier, so that nobody commits the next element's window while
+                // the halo is read; behind a barrier of its own when the zeros of the halo
+                // window were written in the iteration just before (inner == 1).
+                if (inner == 1) lds_barrier();
+                if (active)
+                    for_each_row<TL, CPT, kBwdDepth>(xhalo + pl.row00, [&](int r, const float (&xv)[CPT + 2]) {
+#pragma unroll
+                        for (int cc = 0; cc < 3; ++cc)
+#pragma unroll
+                            for (int c = 0; c < CPT; ++c)
+                                nw[r * 3 + cc][c] = fmaf(xv[c + cc], dsum[c], nw[r * 3 + cc][c]);
+                    });
             }
             lds_barrier();
             if (active) {
@@ -965,10 +994,9 @@ void step_bwd_fast(
         }
         if (pl.slot != 0) return;
     }
-    commit_grads<27, CPT>(dweight, nw, param_mode, neighbour_weight, in_block);
+    commit_grads<27, CPT>(dweight, nw, param_mode, owner_of, always);
     float one[1][CPT];
     auto own_cell = [&](int, int c) { return pl.gc + c; };
-    auto always = [](int, int) { return true; };
 #pragma unroll
     for (int c = 0; c < CPT; ++c) one[0][c] = db[c];
     commit_grads<1, CPT>(dbias, one, param_mode, own_cell, always);
@@ -986,40 +1014,37 @@ void step_bwd_fast(
 }
 
 // ---- backward, second kernel: everything that crosses a block boundary ----------------------
-// The window halo is frozen during the inner iterations, so both the gradient that the cells of
-// NEIGHBOURING blocks receive and the gradient of a weight whose tap reads a halo entry depend
-// on the iterations only through D = sum_i delta_i, which step_bwd_fast leaves in `dsum`.  For a
-// cell c of the block and a tap t with h = c + off_t in another block:
-//   dx[c]    += W[26-t, h] * D[h]        (h's mirrored tap reads c)
-//   dW[t, c] += D[c] * x[h]              (x[h] = 0 outside the grid)
+// The window halo is frozen during the inner iterations, so the gradient that the cells of
+// NEIGHBOURING blocks receive depends on the iterations only through D = sum_i delta_i, which
+// step_bwd_fast leaves in `dsum`.  For a cell c of the block and a tap t with h = c + off_t in
+// another block:
+//   dx[c] += W[26-t, h] * D[h]        (h's mirrored tap reads c)
 // Only boundary cells have such taps, and a tap leaves the block through a face: the work is
 // dealt by FACE.  A slot (one batch element of the block) is 6 faces of bs*bs threads; the
 // thread of face cell c owns the 9 taps that leave through its face, minus those that also
 // leave through a face of a lower axis (edges and corners; counted there).  So every
-// (cell, tap) pair has exactly one thread, which keeps its mirrored weight and its gradient
-// accumulator in registers for the whole batch: 9 of each.  The x window and the D window of
-// the element sit in LDS with their REAL halo (the neighbouring blocks' values, zero outside
-// the grid), two stages alternating, fetched one round ahead.  Every thread leaves what it found
+// (cell, tap) pair has exactly one thread, which keeps its mirrored weight in registers for the
+// whole batch.  The D window of the element sits in LDS with its REAL halo (the neighbouring
+// blocks' values, zero outside the grid), two stages alternating, fetched one round ahead.  Every thread leaves what it found
 // for its cell in a small LDS slab; one round late (after the next barrier) the slot's row
 // threads add the parts of each cell to dx in a fixed order; no atomics.
-// A pass over one element is short (19 LDS reads, 18 FMAs per thread), and a block has few
+// A pass over one element is short (9 LDS reads, 9 FMAs per thread), and a block has few
 // workgroups to hide latency behind: a slot therefore takes E elements per round, so that
 // one barrier, one trip to LDS and one trip to memory serve E elements.
 // LN (the LayerNorm of the network body folded in, see LnFold): when x is the raw output of the
-// step before, the x window holds xhat = (x - mean) * rstd and the affine part is applied as a
-// halo entry is used (its gamma and beta sit in registers beside the pair's weight).  dx as this
-// kernel completes it is the gradient with respect to LayerNorm(x): the row threads, which hold
-// the finished rows, also form the two per-sample sums that LayerNorm's backward needs,
-// sum(gamma dx) and sum(gamma dx xhat), and leave them per 16 lanes.
+// step before, dx as this kernel completes it is the gradient with respect to LayerNorm(x).  The
+// row threads, which hold the finished rows, then also form the two per-sample sums that
+// LayerNorm's backward needs, sum(gamma dx) and sum(gamma dx xhat), and leave them per 16 lanes;
+// for that the x window is fetched as well, as xhat = (x - mean) * rstd.
 template <int BS, int NSLOT, int E, bool LN>
 __global__ __launch_bounds__((6 * BS * BS * NSLOT)) __attribute__((amdgpu_waves_per_eu(3)))
 void step_bwd_cross(
     const float *__restrict__ weight, const float *__restrict__ x, const float *__restrict__ dsum,
-    float *__restrict__ dweight, float *__restrict__ dx, int B, int M, int N, int K, int nblk,
-    int nchunk, int chunk_len, int param_mode, LnFold ln) {
+    float *__restrict__ dx, int B, int M, int N, int K, int nblk, int nchunk, int chunk_len,
+    LnFold ln) {
     using TL = Tile<BS, 1>;  // window geometry only
     constexpr int FS = BS * BS, TPS = 6 * FS;
-    constexpr int PAIR = 2 * TL::WIN;              // [x window | D window] of one element
+    constexpr int PAIR = (LN ? 2 : 1) * TL::WIN;   // [D window | LN: x window] of one element
     constexpr int STAGE = E * PAIR;                // the E elements of a round
     // two stages, two slabs; LN: two more slabs with xhat of the block's own cells, row by row
     constexpr int XROWS = LN ? E * FS * BS : 0;
@@ -1054,8 +1079,7 @@ void step_bwd_cross(
     const bool ri_edge = ri == 0 || ri == BS - 1, rj_edge = rj == 0 || rj == BS - 1;
 
     const bool ln_in = LN && ln.x_stats != nullptr;
-    float vx[9], cw[9];
-    float gh[9], bh[9];     // LN: gamma, beta of the pair's halo cell (1, 0 when x is used as is)
+    float vx[9];
     float grw[BS];  // LN, row threads: gamma of their row
     if (ln_in && is_row) load_cells<BS>(ln.gamma + grow, grw);
     int hoff[9];
@@ -1076,14 +1100,6 @@ void step_bwd_cross(
         hoff[pq] = own + di * TL::PS + dj * TL::RS + dk;
         const long hcell = gcell + (long)(di * N + dj) * K + dk;
         vx[pq] = (mine[pq] && in_grid) ? weight[(26 - t) * cells + hcell] : 0.f;
-        if (LN) {
-            gh[pq] = ln_in ? (in_grid ? ln.gamma[hcell] : 0.f) : 1.f;
-            bh[pq] = (ln_in && in_grid) ? ln.beta[hcell] : 0.f;
-        }
-        // add-in-place mode: slot 0's accumulators start from what the gradient buffer holds
-        cw[pq] = (mine[pq] && param_mode == kParamAddExclusive && slot == 0)
-                     ? dweight[t * cells + gcell]
-                     : 0.f;
     }
     wait_global_loads();
 
@@ -1101,7 +1117,7 @@ void step_bwd_cross(
         for (int e = 0; e < E; ++e) {
             const int sc = min(sample(r, e), s1 - 1);
             const long at = (long)sc * cells;
-            fx.fetch(x + at, px[e]);
+            if (LN) fx.fetch(x + at, px[e]);
             fx.fetch(dsum + at, pd[e]);
             pmean[e] = ln_in ? load_ahead(ln.x_stats, 2 * sc) : 0.f;
             prstd[e] = ln_in ? load_ahead(ln.x_stats, 2 * sc + 1) : 1.f;
@@ -1110,8 +1126,8 @@ void step_bwd_cross(
     auto commit_round = [&](int st) {
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            fx.template commit<1>(stages + st * STAGE + e * PAIR, px[e], pmean[e], prstd[e]);
-            fx.template commit<1>(stages + st * STAGE + e * PAIR + TL::WIN, pd[e]);
+            fx.template commit<1>(stages + st * STAGE + e * PAIR, pd[e]);
+            if (LN) fx.template commit<1>(stages + st * STAGE + e * PAIR + TL::WIN, px[e], pmean[e], prstd[e]);
         }
     };
     float gx[E][BS];  // row threads: dx of their row so far (the own block's part)
@@ -1175,21 +1191,13 @@ void step_bwd_cross(
         fetch_round(r + 1);
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            const float *xw = stages + st * STAGE + e * PAIR, *dw = xw + TL::WIN;
-            const float dc = dw[own];
-            float dh[9], xh[9];
+            const float *dw = stages + st * STAGE + e * PAIR, *xw = dw + TL::WIN;
+            float dh[9];
 #pragma unroll
-            for (int pq = 0; pq < 9; ++pq) {
-                dh[pq] = dw[hoff[pq]];
-                xh[pq] = xw[hoff[pq]];
-            }
-            const bool real = sample(r, e) < s1;
+            for (int pq = 0; pq < 9; ++pq) dh[pq] = dw[hoff[pq]];
             float g = 0.f;
 #pragma unroll
-            for (int pq = 0; pq < 9; ++pq) {
-                g = fmaf(vx[pq], dh[pq], g);
-                cw[pq] = fmaf(real ? dc : 0.f, LN ? fmaf(xh[pq], gh[pq], bh[pq]) : xh[pq], cw[pq]);
-            }
+            for (int pq = 0; pq < 9; ++pq) g = fmaf(vx[pq], dh[pq], g);
             slabs[(st * E + e) * TPS + lane] = g;
             if (ln_in && is_row) {  // xhat of the own row, for the sums one round later
                 float xr[BS];
@@ -1203,35 +1211,6 @@ void step_bwd_cross(
     }
     lds_barrier();
     finish_prev((rounds - 1) & 1);
-
-    if (NSLOT > 1) {
-        float *red = lds;  // NSLOT * TPS floats, reused value by value
-#pragma unroll
-        for (int pq = 0; pq < 9; ++pq) {
-            lds_barrier();
-            red[slot * TPS + lane] = cw[pq];
-            lds_barrier();
-            if (slot == 0) {
-#pragma unroll
-                for (int q = 1; q < NSLOT; ++q) cw[pq] += red[q * TPS + lane];
-            }
-        }
-        if (slot != 0) return;
-    }
-    // every pair is committed, also where its tap reads the zero padding outside the grid (the
-    // gradient is exactly zero and a store-mode caller expects every entry written)
-#pragma unroll
-    for (int pq = 0; pq < 9; ++pq) {
-        const int dp = pq / 3 - 1, dq = pq % 3 - 1;
-        const int di = axis == 0 ? out : dp;
-        const int dj = axis == 0 ? dp : axis == 1 ? out : dq;
-        const int dk = axis == 2 ? out : dq;
-        const int t = (di + 1) * 9 + (dj + 1) * 3 + (dk + 1);
-        if (mine[pq]) {
-            if (param_mode != kParamAtomic) dweight[t * cells + gcell] = cw[pq];
-            else unsafeAtomicAdd(dweight + t * cells + gcell, cw[pq]);
-        }
-    }
 }
 
 __global__ void fill_zero_f32(float *p, long n) {
@@ -1376,15 +1355,13 @@ int launch_bwd_ln(const StepArgs &a, hipStream_t st) {
                        (float *)a.dscale, (float *)a.dx, (float *)a.workspace, a.B, a.M, a.N, a.K,
                        a.inner, p.nblk, p.nchunk, p.chunk_len, param_mode, dx_accumulate, a.ln);
     if (int rc = check_launch("step_bwd_fast")) return rc;
-    // same blocks, same batch chunks, same way of committing parameter gradients (the two
-    // kernels write disjoint entries of dweight)
+    // same blocks, same batch chunks; the parameter gradients are complete, dx is not yet
     constexpr int XSLOT = BS == 8 ? kCrossSlots8 : kCrossSlots4;
     constexpr int XE = BS == 8 ? kCrossElems8 : kCrossElems4;
     hipLaunchKernelGGL((step_bwd_cross<BS, XSLOT, XE, LN>), dim3(padded_grid(p.nblk, p.nchunk)),
                        dim3(6 * BS * BS * XSLOT), 0, st, (const float *)a.weight,
-                       (const float *)a.x, (const float *)a.workspace, (float *)a.dweight,
-                       (float *)a.dx, a.B, a.M, a.N, a.K, p.nblk, p.nchunk, p.chunk_len, param_mode,
-                       a.ln);
+                       (const float *)a.x, (const float *)a.workspace, (float *)a.dx, a.B, a.M, a.N,
+                       a.K, p.nblk, p.nchunk, p.chunk_len, a.ln);
     if (int rc = check_launch("step_bwd_cross")) return rc;
     return GRIDNET_OK;
 }
