@@ -519,16 +519,20 @@ __device__ __forceinline__ float partner_lane(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true));
 }
 
-template <int ACT>
+// LN: the variant with the LayerNorm of the network body folded in, as in step_fwd_fast.
+template <int ACT, bool LN>
 __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(3)))
 void step_fwd_split(
     const float *__restrict__ weight, const float *__restrict__ bias,
     const float *__restrict__ scale, const float *__restrict__ x, float *__restrict__ y, int B, int M,
-    int N, int K, int inner, int nblk, int nchunk, int chunk_len) {
+    int N, int K, int inner, int nblk, int nchunk, int chunk_len, LnFold ln) {
     using TL = Tile<8, 4>;
     using SW = SplitWin;
     using FX = Fetch<TL>;
-    __shared__ __attribute__((aligned(16))) float lds[2 * SW::COPY];
+    // two copies of the window; then, for the folded LayerNorm, gamma and beta laid out alike
+    __shared__ __attribute__((aligned(16))) float lds[(LN ? 4 : 2) * SW::COPY];
+    float *gwin = lds + 2 * SW::COPY, *bwin = gwin + SW::COPY;
+    const bool ln_in = LN && ln.x_stats != nullptr;  // x is the raw output of the step before
 
     int blk, chunk;
     if (!split_block_id(blockIdx.x, nblk, nchunk, blk, chunk)) return;  // grid padding
@@ -577,24 +581,43 @@ void step_fwd_split(
             rv[r] = second ? rt[3 - r] : rt[r];
         }
     }
-    wait_global_loads();
-
-    auto commit = [&](const typename FX::Buf &v) {
+    // A fetched element goes into `copies` window copies at `to`; with `fold` the LayerNorm of
+    // the producer is applied on the way: (v - mean) * rstd * gamma + beta, gamma and beta from
+    // their own windows; entries outside the grid stay zero.
+    auto commit = [&](float *to, int copies, const typename FX::Buf &v, bool fold, float mean, float rstd) {
 #pragma unroll
         for (int e = 0; e < FX::RPT; ++e)
             if (fx.loff[e] >= 0) {
-                const float end = (fx.ok[e] && fx.edge_ok[e]) ? v[e][4] : 0.f;
-                float c[4];
+                float end = v[e][4], c[4];
 #pragma unroll
-                for (int r = 0; r < 4; ++r) c[r] = fx.ok[e] ? (fx.hi[e] ? v[e][3 - r] : v[e][r]) : 0.f;
+                for (int r = 0; r < 4; ++r) c[r] = fx.hi[e] ? v[e][3 - r] : v[e][r];
+                if (LN && fold) {
+                    const float4 g4 = *reinterpret_cast<const float4 *>(gwin + cen_at[e]);
+                    const float4 b4 = *reinterpret_cast<const float4 *>(bwin + cen_at[e]);
+                    c[0] = fmaf((c[0] - mean) * rstd, g4.x, b4.x);
+                    c[1] = fmaf((c[1] - mean) * rstd, g4.y, b4.y);
+                    c[2] = fmaf((c[2] - mean) * rstd, g4.z, b4.z);
+                    c[3] = fmaf((c[3] - mean) * rstd, g4.w, b4.w);
+                    end = fmaf((end - mean) * rstd, gwin[side_at[e]], bwin[side_at[e]]);
+                }
+                if (!(fx.ok[e] && fx.edge_ok[e])) end = 0.f;
 #pragma unroll
-                for (int copy = 0; copy < 2; ++copy) {
-                    *reinterpret_cast<float4 *>(lds + copy * SW::COPY + cen_at[e]) =
+                for (int r = 0; r < 4; ++r) c[r] = fx.ok[e] ? c[r] : 0.f;
+                for (int copy = 0; copy < copies; ++copy) {
+                    *reinterpret_cast<float4 *>(to + copy * SW::COPY + cen_at[e]) =
                         make_float4(c[0], c[1], c[2], c[3]);
-                    lds[copy * SW::COPY + side_at[e]] = end;
+                    to[copy * SW::COPY + side_at[e]] = end;
                 }
             }
     };
+    typename FX::Buf pre;
+    if (ln_in) {  // gamma and beta of the window, once per workgroup
+        fx.fetch(ln.gamma, pre);
+        commit(gwin, 1, pre, false, 0.f, 1.f);
+        fx.fetch(ln.beta, pre);
+        commit(bwin, 1, pre, false, 0.f, 1.f);
+        lds_barrier();
+    }
     auto store_result = [&](int s, const float (&cur)[4]) {
         float out[4];
 #pragma unroll
@@ -603,17 +626,24 @@ void step_fwd_split(
     };
 
     const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
-    typename FX::Buf pre;
-    if (s0 < s1) fx.fetch(x + s0 * cells, pre);
+    float pre_mean = 0.f, pre_rstd = 1.f;  // LayerNorm statistics of the element in `pre`
+    auto fetch_element = [&](int s) {
+        fx.fetch(x + s * cells, pre);
+        if (ln_in) {
+            pre_mean = load_ahead(ln.x_stats, 2 * s);
+            pre_rstd = load_ahead(ln.x_stats, 2 * s + 1);
+        }
+    };
+    if (s0 < s1) fetch_element(s0);
     // The result of an element is stored one element late, after the next window has been
     // committed (see step_fwd_fast).
     float done[4];
     int done_s = -1;
     for (int s = s0; s < s1; ++s) {
-        commit(pre);
+        commit(lds, 2, pre, ln_in, pre_mean, pre_rstd);
         lds_barrier();
         if (done_s >= 0) store_result(done_s, done);
-        if (s + 1 < s1) fx.fetch(x + (s + 1) * cells, pre);  // next element, in flight
+        if (s + 1 < s1) fetch_element(s + 1);  // next element, in flight
         float cur[4];
         {
             const float4 q = *reinterpret_cast<const float4 *>(lds + own);
@@ -645,6 +675,22 @@ void step_fwd_split(
             *reinterpret_cast<float4 *>(lds + ((it + 1) & 1) * SW::COPY + own) =
                 make_float4(cur[0], cur[1], cur[2], cur[3]);
             lds_barrier();
+        }
+        if (LN && ln.y_part) {
+            // statistics of the result for the LayerNorm that follows: every group of 16 lanes
+            // leaves (mean, M2 about that mean) of its 64 cells
+            float sum = 0.f, m2 = 0.f;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sum += cur[r];
+            const float mean = row16_sum(sum) * (1.f / 64);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) m2 = fmaf(cur[r] - mean, cur[r] - mean, m2);
+            m2 = row16_sum(m2);
+            if ((pl.lane & 15) == 0) {
+                float *to = ln.y_part + (((long)s * nblk + blk) * (TL::TPS / 16) + pl.lane / 16) * 2;
+                to[0] = mean;
+                to[1] = m2;
+            }
         }
         done_s = s;
 #pragma unroll
@@ -1035,7 +1081,7 @@ void step_bwd_fast(
 // step before, dx as this kernel completes it is the gradient with respect to LayerNorm(x).  The
 // row threads, which hold the finished rows, then also form the two per-sample sums that
 // LayerNorm's backward needs, sum(gamma dx) and sum(gamma dx xhat), and leave them per 16 lanes;
-// for that the x window is fetched as well, as xhat = (x - mean) * rstd.
+// for that they load their row of x beside their row of dx.
 template <int BS, int NSLOT, int E, bool LN>
 __global__ __launch_bounds__((6 * BS * BS * NSLOT)) __attribute__((amdgpu_waves_per_eu(3)))
 void step_bwd_cross(
@@ -1044,11 +1090,9 @@ void step_bwd_cross(
     LnFold ln) {
     using TL = Tile<BS, 1>;  // window geometry only
     constexpr int FS = BS * BS, TPS = 6 * FS;
-    constexpr int PAIR = (LN ? 2 : 1) * TL::WIN;   // [D window | LN: x window] of one element
+    constexpr int PAIR = TL::WIN;                  // the D window of one element
     constexpr int STAGE = E * PAIR;                // the E elements of a round
-    // two stages, two slabs; LN: two more slabs with xhat of the block's own cells, row by row
-    constexpr int XROWS = LN ? E * FS * BS : 0;
-    constexpr int SLOT = 2 * STAGE + 2 * E * TPS + 2 * XROWS;
+    constexpr int SLOT = 2 * STAGE + 2 * E * TPS;  // two stages, two slabs
     __shared__ __attribute__((aligned(16))) float lds[NSLOT * SLOT];
 
     int blk, chunk;
@@ -1058,7 +1102,6 @@ void step_bwd_cross(
     const int p0 = (blk / (kb * nb)) * BS, q0 = ((blk / kb) % nb) * BS, r0 = (blk % kb) * BS;
     const FetchLines<TL, TPS> fx(lane, p0, q0, r0, M, N, K);
     float *stages = lds + slot * SLOT, *slabs = stages + 2 * STAGE;
-    float *xrows = slabs + 2 * E * TPS;
     const long cells = (long)M * N * K;
 
     // ---- which cell, which taps ----
@@ -1107,8 +1150,7 @@ void step_bwd_cross(
     using Buf = typename FetchLines<TL, TPS>::Buf;
     // element e of round r of this slot; past the end of the chunk it is not `real`
     auto sample = [&](int r, int e) { return s0 + (r * E + e) * NSLOT + slot; };
-    Buf px[E], pd[E];
-    float pmean[E], prstd[E];  // LN: statistics of the elements in px
+    Buf pd[E];
     // Loads and commits are unconditional (past the end of the chunk they repeat its last
     // element, which nobody then uses): with branches around them the compiler cannot count the
     // loads in flight and waits for ALL of them wherever it needs one.
@@ -1117,20 +1159,17 @@ void step_bwd_cross(
         for (int e = 0; e < E; ++e) {
             const int sc = min(sample(r, e), s1 - 1);
             const long at = (long)sc * cells;
-            if (LN) fx.fetch(x + at, px[e]);
             fx.fetch(dsum + at, pd[e]);
-            pmean[e] = ln_in ? load_ahead(ln.x_stats, 2 * sc) : 0.f;
-            prstd[e] = ln_in ? load_ahead(ln.x_stats, 2 * sc + 1) : 1.f;
         }
     };
     auto commit_round = [&](int st) {
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             fx.template commit<1>(stages + st * STAGE + e * PAIR, pd[e]);
-            if (LN) fx.template commit<1>(stages + st * STAGE + e * PAIR + TL::WIN, px[e], pmean[e], prstd[e]);
         }
     };
     float gx[E][BS];  // row threads: dx of their row so far (the own block's part)
+    float xr[E][BS], xmean[E], xrstd[E];  // LN, row threads: their row of x and its statistics
     int r_prev = -1;
     // the round before: its parts are all in slab `st` by now (a barrier lies in between)
     auto finish_prev = [&](int st) {
@@ -1156,13 +1195,12 @@ void step_bwd_cross(
                 }
                 if (s < s1) store_cells<BS>(dx + (long)s * cells + grow, gx[e]);
                 if (ln_in) {
-                    float xh[BS], t1 = 0.f, t2 = 0.f;
-                    load_cells<BS>(xrows + (st * E + e) * FS * BS + lane * BS, xh);
+                    float t1 = 0.f, t2 = 0.f;
 #pragma unroll
                     for (int c = 0; c < BS; ++c) {
                         const float a = grw[c] * gx[e][c];
                         t1 += a;
-                        t2 = fmaf(a, xh[c], t2);
+                        t2 = fmaf(a, (xr[e][c] - xmean[e]) * xrstd[e], t2);
                     }
                     t1 = row16_sum(t1);  // the row threads are whole 16-lane groups
                     t2 = row16_sum(t2);
@@ -1185,13 +1223,20 @@ void step_bwd_cross(
         finish_prev(st ^ 1);
         if (is_row) {  // requested before the prefetch, so that they are awaited first
 #pragma unroll
-            for (int e = 0; e < E; ++e)
-                load_cells<BS>(dx + (long)min(sample(r, e), s1 - 1) * cells + grow, gx[e]);
+            for (int e = 0; e < E; ++e) {
+                const int sc = min(sample(r, e), s1 - 1);
+                load_cells<BS>(dx + (long)sc * cells + grow, gx[e]);
+                if (ln_in) {
+                    load_cells<BS>(x + (long)sc * cells + grow, xr[e]);
+                    xmean[e] = load_ahead(ln.x_stats, 2 * sc);
+                    xrstd[e] = load_ahead(ln.x_stats, 2 * sc + 1);
+                }
+            }
         }
         fetch_round(r + 1);
 #pragma unroll
         for (int e = 0; e < E; ++e) {
-            const float *dw = stages + st * STAGE + e * PAIR, *xw = dw + TL::WIN;
+            const float *dw = stages + st * STAGE + e * PAIR;
             float dh[9];
 #pragma unroll
             for (int pq = 0; pq < 9; ++pq) dh[pq] = dw[hoff[pq]];
@@ -1199,12 +1244,6 @@ void step_bwd_cross(
 #pragma unroll
             for (int pq = 0; pq < 9; ++pq) g = fmaf(vx[pq], dh[pq], g);
             slabs[(st * E + e) * TPS + lane] = g;
-            if (ln_in && is_row) {  // xhat of the own row, for the sums one round later
-                float xr[BS];
-#pragma unroll
-                for (int c = 0; c < BS; ++c) xr[c] = xw[(ri + 1) * TL::PS + (rj + 1) * TL::RS + 1 + c];
-                store_cells<BS>(xrows + (st * E + e) * FS * BS + lane * BS, xr);
-            }
         }
         r_prev = r;
         commit_round(st ^ 1);
@@ -1279,8 +1318,8 @@ template <int BS, int CPT, int NSLOT, int ACT, bool LN> int launch_fwd_ln(const 
                        p.chunk_len, a.ln);
     return check_launch("step_fwd_fast");
 }
-template <int ACT> int launch_fwd_split(const StepArgs &a, hipStream_t st) {
-    auto kern = step_fwd_split<ACT>;
+template <int ACT, bool LN> int launch_fwd_split(const StepArgs &a, hipStream_t st) {
+    auto kern = step_fwd_split<ACT, LN>;
     static int per_cu = 0;
     if (per_cu == 0) {
         int n = 0;
@@ -1291,12 +1330,12 @@ template <int ACT> int launch_fwd_split(const StepArgs &a, hipStream_t st) {
     hipLaunchKernelGGL(kern, dim3(padded_grid(p.nblk, p.nchunk)), dim3(128), 0, st,
                        (const float *)a.weight, (const float *)a.bias, (const float *)a.scale,
                        (const float *)a.x, (float *)a.y, a.B, a.M, a.N, a.K, a.inner, p.nblk, p.nchunk,
-                       p.chunk_len);
+                       p.chunk_len, a.ln);
     return check_launch("step_fwd_split");
 }
 template <int BS, int CPT, int NSLOT, int ACT> int launch_fwd(const StepArgs &a, hipStream_t st) {
+    if (BS == 8) return a.ln.gamma ? launch_fwd_split<ACT, true>(a, st) : launch_fwd_split<ACT, false>(a, st);
     if (a.ln.gamma) return launch_fwd_ln<BS, CPT, NSLOT, ACT, true>(a, st);
-    if (BS == 8) return launch_fwd_split<ACT>(a, st);
     return launch_fwd_ln<BS, CPT, NSLOT, ACT, false>(a, st);
 }
 

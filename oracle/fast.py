@@ -66,7 +66,10 @@ def gridnet_step_fast(
     eps: float = 1e-5,
     normalize: bool = True,
     activation: str = "silu",
+    watch=None,
 ):
+    """``watch``, when given, is called with the pre-activations of every inner iteration (the
+    tests use it to find inputs that keep clear of the kink of relu / leaky_relu)."""
     bs = block_size
     check_step_args(weight, bias, residual_scale, init_activations, bs)
     act = activation_fn(activation)
@@ -76,6 +79,9 @@ def gridnet_step_fast(
     r_blk = to_blocks(residual_scale, bs)
     for _ in range(inner_iterations):
         src = normalise_windows(win, eps) if normalize else win
-        delta = act(pre_activation(src, w_blk, b_blk, bs)) * r_blk
+        u = pre_activation(src, w_blk, b_blk, bs)
+        if watch is not None:
+            watch(u)
+        delta = act(u) * r_blk
         win = win + F.pad(delta, (1,) * 6)
     return from_blocks(win[..., 1:-1, 1:-1, 1:-1])

@@ -11,7 +11,7 @@ import torch
 
 from oracle.network import network_forward, network_forward_backward
 
-from helpers import assert_close
+from helpers import assert_close, inputs_clear_of_kink
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -55,16 +55,26 @@ def oracle(wl, t, backward):
         activation=wl.activation, normalize=wl.normalize)
 
 
-@pytest.mark.parametrize("name,grid,batch,outer", [("C1", 16, 2, 2), ("C3", 32, 3, 3),
-                                                   ("C5", 16, 5, 3), ("C3", 16, 1, 1)])
-def test_fused_chain_matches_oracle(name, grid, batch, outer):
+# leaky_relu (the workloads' own activation) where inputs can be found that keep every
+# pre-activation of the chain clear of its kink, silu at the sizes where they cannot
+@pytest.mark.parametrize("name,grid,batch,outer,activation", [
+    ("C1", 16, 2, 2, None), ("C3", 16, 2, 2, None), ("C5", 16, 1, 2, None), ("C3", 16, 1, 1, None),
+    ("C3", 32, 3, 3, "silu"), ("C5", 16, 5, 3, "silu")])
+def test_fused_chain_matches_oracle(name, grid, batch, outer, activation):
     from gridnet_amd.configs import WORKLOADS, make_inputs
 
     wl = dataclasses.replace(WORKLOADS[name], grid=grid, batch=batch, outer=outer, backward=True)
-    print(f"fused {wl.name} grid={grid} batch={batch} outer={outer}", flush=True)
-    t = randomise_affine(make_inputs(wl))
-    if wl.inner >= 8:  # keep 8 residual updates contractive (fp32 rounding otherwise grows)
-        t["weight"], t["scale"] = t["weight"] * 0.5, t["scale"] * 0.5
+    if activation:
+        wl = dataclasses.replace(wl, activation=activation)
+    print(f"fused {wl.name} grid={grid} batch={batch} outer={outer} act={wl.activation}", flush=True)
+
+    def make(seed):
+        t = randomise_affine(make_inputs(wl, seed=seed))
+        if wl.inner >= 8:  # keep 8 residual updates contractive (fp32 rounding otherwise grows)
+            t["weight"], t["scale"] = t["weight"] * 0.5, t["scale"] * 0.5
+        return t
+
+    t = inputs_clear_of_kink(wl, make)
     for name_, got, exp in zip(NAMES, run_fused(wl, t, True), oracle(wl, t, True)):
         assert_close(got, exp, what=name_)
 
@@ -111,9 +121,12 @@ def test_fused_full_size_agrees_with_op_by_op_chain():
     fused chain."""
     from gridnet_amd.configs import WORKLOADS, make_inputs
 
-    wl = dataclasses.replace(WORKLOADS["C3"], batch=4, outer=3)
+    # silu: with 12 million pre-activations some land within rounding distance of the kink of
+    # leaky_relu, where two fp32 evaluation orders may take different branches and then differ
+    # grossly in the gradients without either being wrong
+    wl = dataclasses.replace(WORKLOADS["C3"], batch=4, outer=3, activation="silu")
     t = randomise_affine(make_inputs(wl))
-    print(f"fused vs op-by-op {wl.name} batch=4 outer=3", flush=True)
+    print(f"fused vs op-by-op {wl.name} batch=4 outer=3 silu", flush=True)
     run_s, d = runner_for(wl, t, True, False)
     ys = run_s.forward(d["x0"]).clone()
     gs = [g.clone() for g in run_s.backward(d["grad_out"])]

@@ -8,7 +8,7 @@ import torch
 
 from oracle.network import network_forward_backward, network_forward
 
-from helpers import assert_close
+from helpers import assert_close, inputs_clear_of_kink
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -48,23 +48,33 @@ def test_c1_exact_config_forward_and_backward():
     from gridnet_amd.configs import WORKLOADS, make_inputs
 
     wl = dataclasses.replace(WORKLOADS["C1"], backward=True)
-    check_against_oracle(wl, make_inputs(wl), True)
+    check_against_oracle(wl, inputs_clear_of_kink(wl, lambda seed: make_inputs(wl, seed=seed)), True)
 
 
-@pytest.mark.parametrize("name,grid,batch,outer", [("C2", 32, 4, 3), ("C3", 32, 3, 3),
-                                                   ("C4", 32, 2, 2), ("C5", 16, 5, 2)])
-def test_workload_shapes_reduced(name, grid, batch, outer):
-    """The benchmark workloads with their own block size, inner depth, bias and activation, on a
+# Gradients are compared under leaky_relu (the workloads' own activation) where inputs can be
+# found that keep every pre-activation of the chain clear of its kink, and under silu at the
+# sizes where they cannot; forward-only workloads need neither (the function is continuous).
+@pytest.mark.parametrize("name,grid,batch,outer,activation", [
+    ("C2", 32, 4, 3, None), ("C4", 32, 2, 2, None),
+    ("C3", 16, 2, 3, None), ("C5", 16, 1, 2, None),
+    ("C3", 32, 3, 3, "silu"), ("C5", 16, 5, 2, "silu")])
+def test_workload_shapes_reduced(name, grid, batch, outer, activation):
+    """The benchmark workloads with their own block size, inner depth and bias, on a
     grid/batch/outer count the CPU oracle finishes in seconds."""
     from gridnet_amd.configs import WORKLOADS, make_inputs
 
     wl = dataclasses.replace(WORKLOADS[name], grid=grid, batch=batch, outer=outer)
-    if wl.inner >= 8:  # keep 8 residual updates contractive (fp32 rounding otherwise grows)
-        t = make_inputs(wl)
-        t["weight"] = t["weight"] * 0.5
-        t["scale"] = t["scale"] * 0.5
-    else:
-        t = make_inputs(wl)
+    if activation:
+        wl = dataclasses.replace(wl, activation=activation)
+
+    def make(seed):
+        t = make_inputs(wl, seed=seed)
+        if wl.inner >= 8:  # keep 8 residual updates contractive (fp32 rounding otherwise grows)
+            t["weight"] = t["weight"] * 0.5
+            t["scale"] = t["scale"] * 0.5
+        return t
+
+    t = inputs_clear_of_kink(wl, make) if wl.backward else make(0)
     check_against_oracle(wl, t, wl.backward)
 
 
@@ -74,7 +84,10 @@ def test_c3_full_grid_one_outer_step():
     from gridnet_amd.configs import WORKLOADS, make_inputs
 
     wl = dataclasses.replace(WORKLOADS["C3"], batch=2, outer=1)
-    check_against_oracle(wl, make_inputs(wl), True)
+    # one step: fp32 rounding moves a pre-activation by ~2e-7, and 2 million of them leave no
+    # room for more than ten times that
+    t = inputs_clear_of_kink(wl, lambda seed: make_inputs(wl, seed=seed), margin=2e-6)
+    check_against_oracle(wl, t, True)
 
 
 def test_c3_full_size_properties():

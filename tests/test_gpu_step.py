@@ -9,7 +9,7 @@ import torch
 from oracle.fast import gridnet_step_fast
 from oracle.manual import gridnet_step_backward_manual
 
-from helpers import ATOL, RTOL, assert_close, make_acts, make_params
+from helpers import ATOL, RTOL, acts_clear_of_kink, assert_close, make_acts, make_params
 
 pytestmark = pytest.mark.gpu
 
@@ -44,7 +44,8 @@ def compare(case, dtype=torch.float32, all_randn=False, rtol=RTOL, atol=ATOL, ba
     w, b, r = make_params(shape, seed=11, dtype=dtype, all_randn=all_randn)
     if inner >= 8:  # keep deep recurrences contractive: fp32 rounding otherwise grows past the bar
         w, r = w * 0.5, r * 0.5
-    x = make_acts(batch, shape, seed=12, dtype=dtype)
+    x = acts_clear_of_kink(w, b, r, batch, shape, inner, bs, 1e-5, normalize, activation, seed=12,
+                           dtype=dtype)
     gy = make_acts(batch, shape, seed=13, dtype=dtype)
     y, grads = run_op(w, b, r, x, gy, inner, bs, 1e-5, normalize, activation)
     ey, egrads = oracle(w, b, r, x, gy, inner, bs, 1e-5, normalize, activation)
