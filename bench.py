@@ -150,10 +150,10 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--workload", default="C3")
-    ap.add_argument("--path", choices=("steps", "fused"), default="steps",
-                    help="steps: one call per step and per LayerNorm, as the reference's callers do "
-                         "(the faster of the two on MI355X as measured); fused: the entry points "
-                         "with the LayerNorm folded into the step kernels")
+    ap.add_argument("--path", choices=("steps", "fused"), default="fused",
+                    help="fused: the entry points with the LayerNorm folded into the step kernels "
+                         "(the faster of the two on MI355X as measured); steps: one call per step "
+                         "and per LayerNorm, as the reference's callers do")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true",
                     help="skip the HIP graph replay (for runs under a counter-collecting profiler)")
@@ -176,7 +176,7 @@ def main():
     traffic = None
     try:
         with open(os.path.join(ROOT, "profiles", "traffic.json")) as fh:
-            traffic = json.load(fh).get(args.workload, {}).get(dominant)
+            traffic = json.load(fh).get(args.workload, {}).get("fused" if fused else "steps", {}).get(dominant)
     except OSError:
         pass
     dom_s = kernel_s[dominant]
