@@ -196,7 +196,9 @@ template <typename TL, int NT = TL::TPS> struct Fetch {  // NT: threads of a slo
     bool ok[RPT];    // the row lies inside the grid
     bool edge_ok[RPT];
     bool hi[RPT];    // second half: [cells..., end entry] instead of [end entry, cells...]
+    int lane0;       // the thread's index in its slot
     __device__ __forceinline__ Fetch(int lane, int p0, int q0, int r0, int M, int N, int K) {
+        lane0 = lane;
 #pragma unroll
         for (int e = 0; e < RPT; ++e) {
             const int id = lane + e * NT;
@@ -248,23 +250,46 @@ template <typename TL, int NT = TL::TPS> struct Fetch {  // NT: threads of a slo
             }
     }
     // The same, with the LayerNorm of the producer applied on the way in: an entry becomes
-    // (v - mean) * rstd * gamma + beta, gamma and beta read from windows `gwin`, `bwin` laid out
-    // like `win`; entries outside the grid stay zero.
-    template <int COPIES = 2>
-    __device__ __forceinline__ void commit_ln(float *win, const Buf &v, const float *gwin,
-                                              const float *bwin, float mean, float rstd) const {
+    // (v - mean) * rstd * gamma + beta; entries outside the grid stay zero.  gamma and beta of a
+    // thread's half rows sit in LDS packed per half row, [gamma cells | beta cells | gamma end,
+    // beta end] at stride GB, so that they come back as three aligned vector reads (read from
+    // windows laid out like `win` they were ten scattered 32-bit reads per half row).
+    static constexpr int GB = (2 * HC + 2 + 3) / 4 * 4;
+    static constexpr int AFFINE = ((NHALF + NT - 1) / NT) * NT * GB;  // floats of the packed table
+    __device__ __forceinline__ void pack_affine(float *gb, const Buf &gam, const Buf &bet) const {
 #pragma unroll
         for (int e = 0; e < RPT; ++e)
             if (loff[e] >= 0) {
+                float *to = gb + (lane0 + e * NT) * GB;
+                float g[HC], b[HC];
+#pragma unroll
+                for (int q = 0; q < HC; ++q) {
+                    g[q] = gam[e][q];
+                    b[q] = bet[e][q];
+                }
+                store_cells<HC>(to, g);
+                store_cells<HC>(to + HC, b);
+                *reinterpret_cast<float2 *>(to + 2 * HC) = make_float2(gam[e][HC], bet[e][HC]);
+            }
+    }
+    template <int COPIES = 2>
+    __device__ __forceinline__ void commit_ln(float *win, const Buf &v, const float *gb, float mean,
+                                              float rstd) const {
+#pragma unroll
+        for (int e = 0; e < RPT; ++e)
+            if (loff[e] >= 0) {
+                const float *from = gb + (lane0 + e * NT) * GB;
+                float g[HC], b[HC];
+                load_cells<HC>(from, g);
+                load_cells<HC>(from + HC, b);
+                const float2 ends = *reinterpret_cast<const float2 *>(from + 2 * HC);
                 const int at_end = loff[e] + (hi[e] ? HC : 0), at_cells = loff[e] + (hi[e] ? 0 : 1);
-                const float end = (ok[e] && edge_ok[e])
-                                      ? fmaf((v[e][HC] - mean) * rstd, gwin[at_end], bwin[at_end])
-                                      : 0.f;
+                const float end = (ok[e] && edge_ok[e]) ? fmaf((v[e][HC] - mean) * rstd, ends.x, ends.y)
+                                                        : 0.f;
                 float val[HC];
 #pragma unroll
                 for (int q = 0; q < HC; ++q)
-                    val[q] = ok[e] ? fmaf((v[e][q] - mean) * rstd, gwin[at_cells + q], bwin[at_cells + q])
-                                   : 0.f;
+                    val[q] = ok[e] ? fmaf((v[e][q] - mean) * rstd, g[q], b[q]) : 0.f;
 #pragma unroll
                 for (int copy = 0; copy < COPIES; ++copy) {
                     win[copy * TL::WIN + at_end] = end;
@@ -398,15 +423,15 @@ void step_fwd_fast(
     const float *__restrict__ scale, const float *__restrict__ x, float *__restrict__ y, int B, int M,
     int N, int K, int inner, int nblk, int nchunk, int chunk_len, LnFold ln) {
     using TL = Tile<BS, CPT>;
-    // per slot two copies of the window; then, for the folded LayerNorm, gamma and beta windows
-    __shared__ __attribute__((aligned(16))) float lds[NSLOT * 2 * TL::WIN + (LN ? 2 * TL::WIN : 0)];
+    // per slot two copies of the window; then, for the folded LayerNorm, the packed gamma/beta
+    __shared__ __attribute__((aligned(16))) float lds[NSLOT * 2 * TL::WIN + (LN ? Fetch<TL>::AFFINE : 0)];
 
     int blk, chunk;
     if (!split_block_id(blockIdx.x, nblk, nchunk, blk, chunk)) return;  // grid padding
     const Place<TL, CPT, NSLOT> pl(threadIdx.x, blk, N, K);
     const Fetch<TL> fx(pl.lane, pl.p0, pl.q0, pl.r0, M, N, K);
     float *win = lds + pl.slot * (2 * TL::WIN);
-    float *gwin = lds + NSLOT * 2 * TL::WIN, *bwin = gwin + TL::WIN;
+    float *affine = lds + NSLOT * 2 * TL::WIN;
     const long cells = (long)M * N * K;
     const bool ln_in = LN && ln.x_stats != nullptr;  // x is the raw output of the step before
 
@@ -418,10 +443,10 @@ void step_fwd_fast(
     typename Fetch<TL>::Buf pre;
     if (ln_in) {  // gamma and beta of the window, once per workgroup
         if (pl.slot == 0) {
+            typename Fetch<TL>::Buf bet;
             fx.fetch(ln.gamma, pre);
-            fx.template commit<1>(gwin, pre);
-            fx.fetch(ln.beta, pre);
-            fx.template commit<1>(bwin, pre);
+            fx.fetch(ln.beta, bet);
+            fx.pack_affine(affine, pre, bet);
         }
         lds_barrier();
     }
@@ -446,7 +471,7 @@ void step_fwd_fast(
         const int s = sb + pl.slot;
         const bool active = s < s1;  // a slot past the end idles through the barriers
         if (active) {
-            if (ln_in) fx.commit_ln(win, pre, gwin, bwin, pre_mean, pre_rstd);
+            if (ln_in) fx.commit_ln(win, pre, affine, pre_mean, pre_rstd);
             else fx.commit(win, pre);
         }
         lds_barrier();
@@ -710,8 +735,8 @@ template <int BS, int CPT> __host__ __device__ constexpr int bwd_slot_floats(int
 }
 // ... and at least the 27 weight planes of the block, which pass through LDS once at set-up
 template <int BS, int CPT, int NSLOT> size_t bwd_lds_bytes(int inner, bool ln = false) {
-    const size_t run = ((size_t)NSLOT * bwd_slot_floats<BS, CPT>(inner) + (ln ? 2 * Tile<BS, CPT>::WIN : 0)) *
-                       sizeof(float);
+    const size_t run = ((size_t)NSLOT * bwd_slot_floats<BS, CPT>(inner) +
+                        (ln ? Fetch<Tile<BS, CPT>>::AFFINE : 0)) * sizeof(float);
     const size_t setup = (size_t)27 * BS * BS * BS * sizeof(float);
     return run > setup ? run : setup;
 }
@@ -766,7 +791,7 @@ void step_bwd_fast(
     // The x window copy that would receive x_inner (never needed) gets zeros in the block's
     // cells instead: the x window's halo alone, for the weights of the taps that read it.
     const float *xhalo = win + (inner & 1) * TL::WIN;
-    float *gwin = lds + NSLOT * slot_floats, *bwin = gwin + TL::WIN;  // LN: gamma, beta windows
+    float *affine = lds + NSLOT * slot_floats;  // LN: gamma and beta of the window, packed
     const long cells = (long)M * N * K;
 
     // nw[t][c] belongs to the weight of the neighbour at c + off_t where that lies in this block,
@@ -831,10 +856,10 @@ void step_bwd_fast(
     }
     typename Fetch<TL>::Buf pre;
     if (ln_in && pl.slot == 0) {  // gamma and beta of the window, once per workgroup
+        typename Fetch<TL>::Buf bet;
         fx.fetch(ln.gamma, pre);
-        fx.template commit<1>(gwin, pre);
-        fx.fetch(ln.beta, pre);
-        fx.template commit<1>(bwin, pre);
+        fx.fetch(ln.beta, bet);
+        fx.pack_affine(affine, pre, bet);
     }
 
     // delta windows: the halo stays zero for the whole kernel
@@ -892,7 +917,7 @@ void step_bwd_fast(
                 g[c] = gnext[c];
             }
         }
-        if (ln_in) fx.commit_ln(win, pre, gwin, bwin, nx_mean, nx_rstd);
+        if (ln_in) fx.commit_ln(win, pre, affine, nx_mean, nx_rstd);
         else fx.commit(win, pre);
     };
     if (ln_in) lds_barrier();  // gamma and beta windows
