@@ -285,7 +285,7 @@ constexpr int kFinUnroll = 4;  // pairs a thread requests before it uses any
 __global__ __launch_bounds__(kFinThreads) void ln_finalize_stats(const float *__restrict__ part,
                                                                  int parts, int count,
                                                                  float *__restrict__ stats, double eps) {
-    __shared__ double red[kFinThreads / kWave];
+    __shared__ double red[kFinThreads / kWave][3];
     const int tid = threadIdx.x, b = blockIdx.x;
     const float2 *ps = reinterpret_cast<const float2 *>(part) + (long)b * parts;
     double s = 0.0, q = 0.0, qm = 0.0;
@@ -305,10 +305,23 @@ __global__ __launch_bounds__(kFinThreads) void ln_finalize_stats(const float *__
             qm += (double)v[k].x * (double)v[k].x;
         }
     }
-    s = block_sum(s, red, tid, kFinThreads);
-    q = block_sum(q, red, tid, kFinThreads);
-    qm = block_sum(qm, red, tid, kFinThreads);
+    // the three sums cross the workgroup together: one trip through LDS, one barrier
+    s = wave_sum(s);
+    q = wave_sum(q);
+    qm = wave_sum(qm);
+    if ((tid & (kWave - 1)) == 0) {
+        red[tid / kWave][0] = s;
+        red[tid / kWave][1] = q;
+        red[tid / kWave][2] = qm;
+    }
+    __syncthreads();
     if (tid == 0) {
+        s = q = qm = 0.0;
+        for (int w = 0; w < kFinThreads / kWave; ++w) {
+            s += red[w][0];
+            q += red[w][1];
+            qm += red[w][2];
+        }
         const double mean = s / parts;
         // sum count (mean_i - mean)^2 = count (sum mean_i^2 - parts mean^2)
         const double var = (q + count * (qm - parts * mean * mean)) / ((double)parts * count);
@@ -321,7 +334,7 @@ __global__ __launch_bounds__(kFinThreads) void ln_finalize_stats(const float *__
 __global__ __launch_bounds__(kFinThreads) void ln_finalize_sums(const float *__restrict__ part,
                                                                 int parts, long n,
                                                                 float *__restrict__ sums) {
-    __shared__ double red[kFinThreads / kWave];
+    __shared__ double red[kFinThreads / kWave][2];
     const int tid = threadIdx.x, b = blockIdx.x;
     const float2 *ps = reinterpret_cast<const float2 *>(part) + (long)b * parts;
     double s1 = 0.0, s2 = 0.0;
@@ -338,9 +351,19 @@ __global__ __launch_bounds__(kFinThreads) void ln_finalize_sums(const float *__r
             s2 += (double)v[k].y;
         }
     }
-    s1 = block_sum(s1, red, tid, kFinThreads);
-    s2 = block_sum(s2, red, tid, kFinThreads);
+    s1 = wave_sum(s1);
+    s2 = wave_sum(s2);
+    if ((tid & (kWave - 1)) == 0) {
+        red[tid / kWave][0] = s1;
+        red[tid / kWave][1] = s2;
+    }
+    __syncthreads();
     if (tid == 0) {
+        s1 = s2 = 0.0;
+        for (int w = 0; w < kFinThreads / kWave; ++w) {
+            s1 += red[w][0];
+            s2 += red[w][1];
+        }
         sums[2 * b] = (float)(s1 / (double)n);
         sums[2 * b + 1] = (float)(s2 / (double)n);
     }
