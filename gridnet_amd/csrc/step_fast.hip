@@ -25,11 +25,14 @@
 //     of the NEIGHBOUR's mirrored weight W[26-t, c + off_t], and this thread is the only one that
 //     ever contributes to it, so it accumulates in a register over iterations and batch elements
 //     (the x window is not re-read in the reverse sweep);
-//   * everything that crosses a block boundary -- what the cells of NEIGHBOURING blocks receive,
-//     and the gradient of a weight whose tap reads a (frozen) halo entry -- depends on the
-//     iterations only through D = sum_i delta_i.  The first kernel leaves D of every cell in a
-//     scratch tensor and a second kernel (step_bwd_cross), dealt by block face, works both out
-//     from the D and x windows with their real halo and completes dx, in a fixed order.
+//   * what depends on a (frozen) halo entry or on another block depends on the iterations only
+//     through D = sum_i delta_i.  The gradient of a weight whose tap reads a halo entry is
+//     x_halo * D: the first kernel adds it once per element.  What the cells of NEIGHBOURING
+//     blocks receive needs the neighbours' D: the first kernel leaves D of every cell in a
+//     scratch tensor and a second kernel (step_bwd_cross), dealt by block face, works it out
+//     from the D window with its real halo and completes dx, in a fixed order.
+// Forward with 8^3 blocks: the same mapping over a window stored in two parts, so that every LDS
+// access of the inner loop is aligned and free of bank conflicts (step_fwd_split).
 // Parameter gradients leave the kernel once per workgroup: reduced across slots through LDS and,
 // when one workgroup owns the whole batch of its block, written with plain stores.  Results are
 // bitwise reproducible in that case.
