@@ -52,6 +52,11 @@ def test_host_only_entry_points():
     assert native.last_error() == "cannot backprop through more than 32 inner iterations"
     rc = native.lib.gridnet_hip_forward(0, 8, 8, 8, 8, 8, 2, 8, 8, 8, 1, 8, 1e-5, 0, 7, None)
     assert rc == 2 and "unknown activation function" in native.last_error()
+    # 32-bit cell indexing inside a sample: 27 * 432^3 is past 2^31, 27 * 424^3 is not
+    rc = native.lib.gridnet_hip_forward(0, 8, 8, 8, 8, 8, 1, 432, 432, 432, 1, 8, 1e-5, 0, 0, None)
+    assert rc == 1 and "grid too large" in native.last_error()
+    rc = native.lib.gridnet_hip_forward(0, None, 8, 8, 8, 8, 1, 424, 424, 424, 1, 8, 1e-5, 0, 0, None)
+    assert rc == 1 and "null input pointer" in native.last_error()
     assert native.lib.gridnet_hip_layernorm_workspace_bytes(0, 32, 64 ** 3) == (32 * 64 * 2 + 64) * 4
     rc = native.lib.gridnet_hip_layernorm_forward(0, 8, 8, 8, 8, 8, 8, 4, 4096, 1e-5, None, 0, None)
     assert rc == 4 and "workspace" in native.last_error()

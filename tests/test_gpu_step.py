@@ -179,3 +179,61 @@ def test_dispatcher_takes_the_hip_path():
     ey = gridnet_step_fast(w.cpu().double(), b.cpu().double(), r.cpu().double(), x.cpu().double(),
                            2, 8, 1e-5, False, "leaky_relu")
     assert_close(y, ey, what="y")
+
+
+@pytest.mark.parametrize("bs", [8, 4])
+def test_largest_grid_the_index_range_allows(bs):
+    """424^3 cells: 27 * M * N * K is 4 % below 2^31 (the bound of the 32-bit cell indexing
+    inside a sample), and 53^3 = 148 877 blocks (106^3 of side 4) is more than the reference's launch
+    geometry can address (gridDim.y <= 65 535, src/gridnet_cuda_kernels.cu:751).  Too large for
+    the CPU oracle, so the result is held to the closed form that the oracle tests pin on small
+    grids: with positive data relu is the identity with derivative 1, and one inner iteration
+    does not depend on the blocks, so with w = 0 except tap 26 = 1
+        y = x + r (b + S26 x),   dx = dy + S26^T (r dy),   dW[t] = r dy St x,   db = r dy,
+        dr = dy (b + S26 x)
+    where St x is x shifted by tap t's offset with zeros outside the grid."""
+    import gc
+
+    from gridnet_amd.backend_cuda import GridnetCudaOp
+
+    g = 424
+    shape = (g, g, g)
+    print(f"largest grid {shape} bs={bs}", flush=True)
+    gen = torch.Generator(device=DEV).manual_seed(5)
+    w = torch.zeros(27, *shape, device=DEV)
+    w[26] = 1.0
+    b = torch.rand(shape, device=DEV, generator=gen) + 0.1
+    r = torch.rand(shape, device=DEV, generator=gen) + 0.5
+    x = torch.rand(1, *shape, device=DEV, generator=gen) + 0.1
+    dy = torch.randn(1, *shape, device=DEV, generator=gen)
+
+    def shifted(v, t):  # v[c + off_t], zero outside the grid
+        da, db_, dc = t // 9 - 1, (t // 3) % 3 - 1, t % 3 - 1
+        out = torch.zeros_like(v)
+        src = [slice(max(d, 0), g + min(d, 0)) for d in (da, db_, dc)]
+        dst = [slice(max(-d, 0), g + min(-d, 0)) for d in (da, db_, dc)]
+        out[(..., *dst)] = v[(..., *src)]
+        return out
+
+    leaves = [t.requires_grad_(True) for t in (w, b, r, x)]
+    y = GridnetCudaOp.apply(*leaves, 1, bs, 1e-5, False, "relu")
+    dw, db, dr, dx = torch.autograd.grad(y, leaves, dy)
+    u = b + shifted(x, 26)[0]
+    assert_close(y[0, ::7, ::5, ::3], (x[0] + r * u)[::7, ::5, ::3], what="y")
+    assert_close(y[0, -1, -1, :], (x[0] + r * u)[-1, -1, :], what="y, last row")  # S26 x = 0 there
+    delta = (r * dy[0]).detach()
+    assert_close(db[::7, ::5, ::3], delta[::7, ::5, ::3], what="dbias")
+    assert_close(dr[::7, ::5, ::3], (dy[0] * u).detach()[::7, ::5, ::3], what="dscale")
+    back = torch.zeros_like(delta)
+    back[1:, 1:, 1:] = delta[:-1, :-1, :-1]  # S26^T
+    assert_close(dx[0, ::7, ::5, ::3], (dy[0] + back)[::7, ::5, ::3], what="dx")
+    del back, u
+    for t in (0, 1, 13, 25, 26):  # both ends of the plane range, the centre, two more
+        want = delta * shifted(x.detach(), t)[0]
+        assert_close(dw[t, ::7, ::5, ::3], want[::7, ::5, ::3], what=f"dweight[{t}]")
+        # whole planes at the far corner, where the linear index is largest
+        assert_close(dw[t, -16:, -16:, -16:], want[-16:, -16:, -16:], what=f"dweight[{t}] corner")
+        del want
+    del w, dw, leaves, y
+    gc.collect()
+    torch.cuda.empty_cache()
