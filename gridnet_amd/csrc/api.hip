@@ -64,7 +64,7 @@ using namespace gridnet;
 
 extern "C" {
 
-int gridnet_hip_version(void) { return 2; }  // 2: fused body entry points
+int gridnet_hip_version(void) { return 3; }  // 2: fused body entry points; 3: residual forward
 
 const char *gridnet_hip_last_error(void) { return error_buffer(); }
 
@@ -239,11 +239,11 @@ size_t gridnet_hip_fused_workspace_bytes(int B, int M, int N, int K, int inner, 
     return fused_backward_dsum(a) + fused_backward_parts(a);
 }
 
-int gridnet_hip_fused_forward(int dtype, const void *weight, const void *bias, const void *scale,
-                              const void *gamma, const void *beta, const void *x,
-                              const void *x_stats, void *y_raw, void *y_stats, int B, int M, int N,
-                              int K, int inner, int block_size, double ln_eps, int activation,
-                              void *workspace, size_t workspace_bytes, void *stream) {
+static int fused_forward(int dtype, const void *weight, const void *bias, const void *scale,
+                         const void *gamma, const void *beta, const void *x, const void *x_stats,
+                         void *y_raw, void *y_stats, int B, int M, int N, int K, int inner,
+                         int block_size, double ln_eps, int activation, void *workspace,
+                         size_t workspace_bytes, void *stream, int residual) {
     StepArgs a{};
     a.dtype = dtype; a.weight = weight; a.bias = bias; a.scale = scale; a.x = x; a.y = y_raw;
     a.B = B; a.M = M; a.N = N; a.K = K; a.inner = inner; a.block_size = block_size;
@@ -251,6 +251,8 @@ int gridnet_hip_fused_forward(int dtype, const void *weight, const void *bias, c
     if (int rc = check_fused(a, false)) return rc;
     if (B == 0) return GRIDNET_OK;
     if (!gamma || !beta || !y_stats) return fail(GRIDNET_ERR_ARGUMENT, "null pointer");
+    if (residual && !x_stats)
+        return fail(GRIDNET_ERR_ARGUMENT, "the residual form normalises its input: x_stats is required");
     const size_t need = fused_forward_workspace(a);
     if (!workspace || workspace_bytes < need)
         return fail(GRIDNET_ERR_WORKSPACE, "fused forward needs %zu bytes of workspace, got %zu", need,
@@ -260,11 +262,31 @@ int gridnet_hip_fused_forward(int dtype, const void *weight, const void *bias, c
     a.ln.beta = (const float *)beta;
     a.ln.x_stats = (const float *)x_stats;
     a.ln.y_part = (float *)workspace;
+    a.ln.residual = residual;
     if (int rc = step_forward_fast(a, st)) return rc;
     const int nblk = (M / block_size) * (N / block_size) * (K / block_size);
     return layernorm_finalize_stats((const float *)workspace, nblk * step_fast_forward_parts(block_size),
                                     step_fast_forward_part_count(block_size), (float *)y_stats, B,
                                     ln_eps, st);
+}
+
+int gridnet_hip_fused_forward(int dtype, const void *weight, const void *bias, const void *scale,
+                              const void *gamma, const void *beta, const void *x,
+                              const void *x_stats, void *y_raw, void *y_stats, int B, int M, int N,
+                              int K, int inner, int block_size, double ln_eps, int activation,
+                              void *workspace, size_t workspace_bytes, void *stream) {
+    return fused_forward(dtype, weight, bias, scale, gamma, beta, x, x_stats, y_raw, y_stats, B, M, N,
+                         K, inner, block_size, ln_eps, activation, workspace, workspace_bytes, stream, 0);
+}
+
+int gridnet_hip_fused_forward_residual(int dtype, const void *weight, const void *bias,
+                                       const void *scale, const void *gamma, const void *beta,
+                                       const void *x, const void *x_stats, void *y, void *y_stats,
+                                       int B, int M, int N, int K, int inner, int block_size,
+                                       double ln_eps, int activation, void *workspace,
+                                       size_t workspace_bytes, void *stream) {
+    return fused_forward(dtype, weight, bias, scale, gamma, beta, x, x_stats, y, y_stats, B, M, N, K,
+                         inner, block_size, ln_eps, activation, workspace, workspace_bytes, stream, 1);
 }
 
 int gridnet_hip_layernorm_apply(int dtype, const void *x, const void *stats, const void *gamma,

@@ -24,6 +24,9 @@ struct LnFold {
     const float *y_sums;        // [B,2]: mean(g), mean(g * yhat) with g = gamma * incoming gradient
     float *dgamma, *dbeta;      // [M,N,K], summed over the batch, committed like dbias
     float *x_part;              // partial sums for the LayerNorm backward of x: [B, nblk, parts, 2]
+    // forward only: the output is x + (step(LayerNorm(x)) - LayerNorm(x)), the reference's
+    // outer_residual form (gridnet/scripts/train_imagenet.py:81-83); needs x_stats
+    int residual;
 };
 
 struct StepArgs {

@@ -419,7 +419,10 @@ constexpr int kFwdDepth = 9;  // neighbour rows requested ahead of the arithmeti
 
 // LN: the variant with the LayerNorm of the network body folded in (see LnFold); without it
 // `ln` is ignored and the code is the plain step's.
-template <int BS, int CPT, int NSLOT, int ACT, bool LN>
+// RES (with LN): the output is x + (result - LayerNorm(x)), the reference's outer_residual form
+// (gridnet/scripts/train_imagenet.py:81-83); the statistics left for the next LayerNorm are
+// those of that output.
+template <int BS, int CPT, int NSLOT, int ACT, bool LN, bool RES = false>
 __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) __attribute__((amdgpu_waves_per_eu(3)))
 void step_fwd_fast(
     const float *__restrict__ weight, const float *__restrict__ bias,
@@ -480,10 +483,15 @@ void step_fwd_fast(
         lds_barrier();
         if (done_s >= 0) store_cells<CPT>(y + done_s * cells + pl.gc, done);
         if (s + NSLOT < s1) fetch_element(s + NSLOT);  // next element, in flight
-        float cur[CPT];
+        float cur[CPT], base[CPT], raw[CPT];
         if (active) {
 #pragma unroll
             for (int c = 0; c < CPT; ++c) cur[c] = win[pl.own + c];
+            if (RES) {
+                load_cells<CPT>(x + s * cells + pl.gc, raw);
+#pragma unroll
+                for (int c = 0; c < CPT; ++c) base[c] = cur[c];
+            }
         }
         for (int it = 0; it < inner; ++it) {
             if (active) {
@@ -496,6 +504,10 @@ void step_fwd_fast(
                 }
             }
             lds_barrier();
+        }
+        if (RES && active) {
+#pragma unroll
+            for (int c = 0; c < CPT; ++c) cur[c] = raw[c] + (cur[c] - base[c]);
         }
         if (LN && active && ln.y_part) {
             // statistics of the result for the LayerNorm that follows: every group of 16 lanes
@@ -547,8 +559,8 @@ __device__ __forceinline__ float partner_lane(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xf, 0xf, true));
 }
 
-// LN: the variant with the LayerNorm of the network body folded in, as in step_fwd_fast.
-template <int ACT, bool LN>
+// LN, RES: the variants with the LayerNorm of the network body folded in, as in step_fwd_fast.
+template <int ACT, bool LN, bool RES = false>
 __global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(3)))
 void step_fwd_split(
     const float *__restrict__ weight, const float *__restrict__ bias,
@@ -672,10 +684,19 @@ void step_fwd_split(
         lds_barrier();
         if (done_s >= 0) store_result(done_s, done);
         if (s + 1 < s1) fetch_element(s + 1);  // next element, in flight
-        float cur[4];
+        float cur[4], base[4], raw[4];
         {
             const float4 q = *reinterpret_cast<const float4 *>(lds + own);
             cur[0] = q.x; cur[1] = q.y; cur[2] = q.z; cur[3] = q.w;
+        }
+        if (RES) {  // the raw input of the owned cells, in register order like `cur`
+            float rt[4];
+            load_cells<4>(x + s * cells + pl.gc, rt);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                raw[r] = second ? rt[3 - r] : rt[r];
+                base[r] = cur[r];
+            }
         }
         for (int it = 0; it < inner; ++it) {
             const float *from = lds + (it & 1) * SW::COPY;
@@ -703,6 +724,10 @@ void step_fwd_split(
             *reinterpret_cast<float4 *>(lds + ((it + 1) & 1) * SW::COPY + own) =
                 make_float4(cur[0], cur[1], cur[2], cur[3]);
             lds_barrier();
+        }
+        if (RES) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) cur[r] = raw[r] + (cur[r] - base[r]);
         }
         if (LN && ln.y_part) {
             // statistics of the result for the LayerNorm that follows: every group of 16 lanes
@@ -1328,9 +1353,10 @@ Plan make_plan(const StepArgs &a, int nslot, int resident, bool whole_batch_per_
     return p;
 }
 
-template <int BS, int CPT, int NSLOT, int ACT, bool LN> int launch_fwd_ln(const StepArgs &a, hipStream_t st) {
+template <int BS, int CPT, int NSLOT, int ACT, bool LN, bool RES = false>
+int launch_fwd_ln(const StepArgs &a, hipStream_t st) {
     using TL = Tile<BS, CPT>;
-    auto kern = step_fwd_fast<BS, CPT, NSLOT, ACT, LN>;
+    auto kern = step_fwd_fast<BS, CPT, NSLOT, ACT, LN, RES>;
     static int per_cu = 0;
     if (per_cu == 0) {
         int n = 0;
@@ -1346,8 +1372,8 @@ template <int BS, int CPT, int NSLOT, int ACT, bool LN> int launch_fwd_ln(const 
                        p.chunk_len, a.ln);
     return check_launch("step_fwd_fast");
 }
-template <int ACT, bool LN> int launch_fwd_split(const StepArgs &a, hipStream_t st) {
-    auto kern = step_fwd_split<ACT, LN>;
+template <int ACT, bool LN, bool RES = false> int launch_fwd_split(const StepArgs &a, hipStream_t st) {
+    auto kern = step_fwd_split<ACT, LN, RES>;
     static int per_cu = 0;
     if (per_cu == 0) {
         int n = 0;
@@ -1362,6 +1388,10 @@ template <int ACT, bool LN> int launch_fwd_split(const StepArgs &a, hipStream_t 
     return check_launch("step_fwd_split");
 }
 template <int BS, int CPT, int NSLOT, int ACT> int launch_fwd(const StepArgs &a, hipStream_t st) {
+    if (a.ln.gamma && a.ln.residual) {
+        if (BS == 8) return launch_fwd_split<ACT, true, true>(a, st);
+        return launch_fwd_ln<BS, CPT, NSLOT, ACT, true, true>(a, st);
+    }
     if (BS == 8) return a.ln.gamma ? launch_fwd_split<ACT, true>(a, st) : launch_fwd_split<ACT, false>(a, st);
     if (a.ln.gamma) return launch_fwd_ln<BS, CPT, NSLOT, ACT, true>(a, st);
     return launch_fwd_ln<BS, CPT, NSLOT, ACT, false>(a, st);

@@ -34,6 +34,7 @@ EXPORTS = (
     "gridnet_hip_layernorm_backward",
     "gridnet_hip_fused_workspace_bytes",
     "gridnet_hip_fused_forward",
+    "gridnet_hip_fused_forward_residual",
     "gridnet_hip_layernorm_apply",
     "gridnet_hip_layernorm_backward_sums",
     "gridnet_hip_fused_backward",
@@ -79,6 +80,8 @@ def _load():
     lib.gridnet_hip_fused_forward.restype = i
     lib.gridnet_hip_fused_forward.argtypes = [i, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, d, i,
                                               p, z, p]
+    lib.gridnet_hip_fused_forward_residual.restype = i
+    lib.gridnet_hip_fused_forward_residual.argtypes = lib.gridnet_hip_fused_forward.argtypes
     lib.gridnet_hip_layernorm_apply.restype = i
     lib.gridnet_hip_layernorm_apply.argtypes = [i, p, p, p, p, p, i, l, p]
     lib.gridnet_hip_layernorm_backward_sums.restype = i

@@ -9,6 +9,10 @@ memory.  Order of operations: gridnet/scripts/train_mnist.py:62-64.
 step kernels: a step reads the raw output of the step before it and normalises it while
 loading, so the LayerNorm costs no pass over the activations of its own (one, for the final
 output).  Same results within rounding; fp32, ``normalize=False``, ``inner >= 1`` only.
+
+``outer_residual=True`` is the other shape of the loop, ``n = norm(h); h = h + (net(n) - n)``
+(gridnet/scripts/train_imagenet.py:81-83), through the fused forward entry point made for it;
+forward only (the autograd module ``GridnetBody`` trains this shape).
 """
 
 import torch
@@ -20,7 +24,7 @@ class BodyRunner:
     def __init__(self, weight, bias, scale, gamma, beta, batch: int, inner: int, outer: int,
                  block_size: int, activation: str = "leaky_relu", normalize: bool = False,
                  eps: float = 1e-5, ln_eps: float = 1e-5, backward: bool = True,
-                 fused: bool = False):
+                 fused: bool = False, outer_residual: bool = False):
         self.w, self.b, self.r, self.gamma, self.beta = weight, bias, scale, gamma, beta
         self.B, (self.M, self.N, self.K) = batch, bias.shape
         self.inner, self.outer, self.bs = inner, outer, block_size
@@ -53,6 +57,10 @@ class BodyRunner:
             self.bw_ws = _n.workspace(self.bw_ws_bytes, dev)
         self.on_launch = None  # optional hook(name, phase) for per-kernel timing
         self.fused = fused
+        self.outer_residual = outer_residual
+        if outer_residual and (backward or not fused):
+            raise RuntimeError("outer_residual runs through the fused forward entry point only "
+                               "(fused=True, backward=False); GridnetBody trains this shape")
         if fused:
             if weight.dtype != torch.float32 or normalize or inner < 1:
                 raise RuntimeError("the fused body covers float32, normalize=False, inner >= 1")
@@ -113,6 +121,27 @@ class BodyRunner:
         self._mark("ln_fwd", 1)
         return out
 
+    def _residual_forward(self, x0):
+        """h = h + (net(norm(h)) - norm(h)), ``outer`` times; returns the last h as it is."""
+        stream = _n.current_stream(self.w)
+        # statistics of the first input: the LayerNorm entry point's, its output unused
+        self.norm_forward(x0, self.s[0], 0, stream)
+        self.stats[0, :, 0].copy_(self.mean[0])
+        self.stats[0, :, 1].copy_(self.rstd[0])
+        h, stats = x0, self.stats[0]
+        for j in range(self.outer):
+            out = (self.s[0], self.h[1])[j % 2]
+            out_stats = self.stats[(j + 1) % 2]
+            self._mark("step_fwd", 0)
+            _n.check(_n.lib.gridnet_hip_fused_forward_residual(
+                self.dt, self.w.data_ptr(), self.b.data_ptr(), self.r.data_ptr(),
+                self.gamma.data_ptr(), self.beta.data_ptr(), h.data_ptr(), stats.data_ptr(),
+                out.data_ptr(), out_stats.data_ptr(), self.B, self.M, self.N, self.K, self.inner,
+                self.bs, self.ln_eps, self.act, self.fw_ws.data_ptr(), self.fw_ws_bytes, stream))
+            self._mark("step_fwd", 1)
+            h, stats = out, out_stats
+        return h
+
     def _fused_backward(self, grad_out):
         stream = _n.current_stream(self.w)
         last = self.outer - 1
@@ -143,6 +172,8 @@ class BodyRunner:
 
     def forward(self, x0):
         """Returns the buffer holding the result (valid until the next call)."""
+        if self.outer_residual:
+            return self._residual_forward(x0)
         if self.fused:
             return self._fused_forward(x0)
         stream = _n.current_stream(self.w)

@@ -158,6 +158,19 @@ int gridnet_hip_fused_forward(int dtype, const void *weight, const void *bias, c
                               int K, int inner, int block_size, double ln_eps, int activation,
                               void *workspace, size_t workspace_bytes, void *stream);
 
+/* The reference's outer_residual form of one outer step, forward only
+ * (gridnet/scripts/train_imagenet.py:81-83: n = norm(h); h = h + (net(n) - n)):
+ * y = x + (step(n) - n) with n = LayerNorm(x; x_stats, gamma, beta), y_stats = statistics of y,
+ * which the next step of such a chain takes as its x_stats.  x_stats is required (the
+ * statistics of the chain's first input come from gridnet_hip_layernorm_forward).  The result of
+ * a chain is the y of its last step as it is.  Workspace as for gridnet_hip_fused_forward. */
+int gridnet_hip_fused_forward_residual(int dtype, const void *weight, const void *bias,
+                                       const void *scale, const void *gamma, const void *beta,
+                                       const void *x, const void *x_stats, void *y, void *y_stats,
+                                       int B, int M, int N, int K, int inner, int block_size,
+                                       double ln_eps, int activation, void *workspace,
+                                       size_t workspace_bytes, void *stream);
+
 /* y = (x - mean) * rstd * gamma + beta with statistics that are already known: the LayerNorm
  * after the LAST step of a chain, whose output is needed as a tensor. */
 int gridnet_hip_layernorm_apply(int dtype, const void *x, const void *stats, const void *gamma,

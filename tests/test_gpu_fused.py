@@ -90,6 +90,30 @@ def test_fused_forward_only_matches_oracle(name, grid, batch, outer):
     assert_close(got, exp, what="y")
 
 
+@pytest.mark.parametrize("name,grid,batch,outer", [("C3", 32, 3, 3), ("C5", 16, 5, 3), ("C2", 16, 2, 1)])
+def test_fused_residual_forward_matches_oracle(name, grid, batch, outer):
+    """The outer_residual shape of the loop, n = norm(h); h = h + (net(n) - n)
+    (gridnet/scripts/train_imagenet.py:81-83), through gridnet_hip_fused_forward_residual."""
+    from gridnet_amd.configs import WORKLOADS, make_inputs
+    from gridnet_amd.runner import BodyRunner
+
+    wl = dataclasses.replace(WORKLOADS[name], grid=grid, batch=batch, outer=outer, backward=False)
+    print(f"fused residual forward {wl.name} grid={grid} batch={batch} outer={outer}", flush=True)
+    t = randomise_affine(make_inputs(wl))
+    if wl.inner >= 8:
+        t["weight"], t["scale"] = t["weight"] * 0.5, t["scale"] * 0.5
+    d = {k: v.to(DEV) for k, v in t.items()}
+    run = BodyRunner(d["weight"], d["bias"], d["scale"], d["gamma"], d["beta"], batch, wl.inner,
+                     wl.outer, wl.block_size, wl.activation, wl.normalize, backward=False,
+                     fused=True, outer_residual=True)
+    got = run.forward(d["x0"]).clone()
+    exp = network_forward(*[t[k].double() for k in PARAMS], t["x0"].double(), wl.inner, wl.outer,
+                          wl.block_size, wl.activation, wl.normalize, outer_residual=True)
+    # the result is not normalised: values grow with the number of outer steps
+    assert_close(got, exp, what="h")
+    assert torch.equal(d["x0"].cpu(), t["x0"]), "the input was modified"
+
+
 @pytest.mark.parametrize("shape", [(8, 16, 24), (24, 8, 16)])
 def test_fused_chain_non_cubic_grid(shape):
     """Axes of different lengths: catches a swapped stride in the window, face or row indexing."""
