@@ -64,7 +64,7 @@ using namespace gridnet;
 
 extern "C" {
 
-int gridnet_hip_version(void) { return 3; }  // 2: fused body entry points; 3: residual forward
+int gridnet_hip_version(void) { return 3; }  // 2: fused body entry points; 3: residual forward and backward
 
 const char *gridnet_hip_last_error(void) { return error_buffer(); }
 
@@ -317,13 +317,14 @@ int gridnet_hip_layernorm_backward_sums(int dtype, const void *dy, const void *x
                                    (hipStream_t)stream);
 }
 
-int gridnet_hip_fused_backward(int dtype, const void *weight, const void *bias, const void *scale,
-                               const void *gamma, const void *beta, const void *x,
-                               const void *x_stats, const void *dy, const void *y_raw,
-                               const void *y_stats, const void *y_sums, void *dweight, void *dbias,
-                               void *dscale, void *dgamma, void *dbeta, void *dx, void *x_sums, int B,
-                               int M, int N, int K, int inner, int block_size, int activation,
-                               int flags, void *workspace, size_t workspace_bytes, void *stream) {
+static int fused_backward(int dtype, const void *weight, const void *bias, const void *scale,
+                          const void *gamma, const void *beta, const void *x, const void *x_stats,
+                          const void *dy, const void *y_raw, const void *y_stats, const void *y_sums,
+                          void *dweight, void *dbias, void *dscale, void *dgamma, void *dbeta,
+                          void *dx, void *x_sums, int B, int M, int N, int K, int inner,
+                          int block_size, int activation, int flags, void *workspace,
+                          size_t workspace_bytes, void *stream, int residual, const void *g_prev,
+                          void *g_out) {
     StepArgs a{};
     a.dtype = dtype; a.weight = weight; a.bias = bias; a.scale = scale; a.x = x; a.dy = dy;
     a.dweight = dweight; a.dbias = dbias; a.dscale = dscale; a.dx = dx;
@@ -333,8 +334,18 @@ int gridnet_hip_fused_backward(int dtype, const void *weight, const void *bias, 
     a.ln.gamma = (const float *)gamma;  // before the checks: the LDS budget depends on it
     if (int rc = check_fused(a, true)) return rc;
     if (B == 0) return GRIDNET_OK;
-    if (!gamma || !beta || !y_raw || !y_stats || !y_sums || !dgamma || !dbeta)
-        return fail(GRIDNET_ERR_ARGUMENT, "null pointer");
+    if (!gamma || !beta || !dgamma || !dbeta) return fail(GRIDNET_ERR_ARGUMENT, "null pointer");
+    if (!residual) {
+        if (!y_raw || !y_stats || !y_sums) return fail(GRIDNET_ERR_ARGUMENT, "null pointer");
+    } else {
+        // the last step of a chain is handed G' itself; every other one forms it
+        const bool given = !y_raw;
+        if (given ? (y_stats || y_sums || g_prev || g_out) : (!y_stats || !y_sums || !g_prev || !g_out))
+            return fail(GRIDNET_ERR_ARGUMENT,
+                        "y_raw, y_stats, y_sums, g_prev and g_out go together: all or none");
+        if (!x_stats)
+            return fail(GRIDNET_ERR_ARGUMENT, "the residual form normalises its input: x_stats is required");
+    }
     if ((x_stats == nullptr) != (x_sums == nullptr))
         return fail(GRIDNET_ERR_ARGUMENT, "x_stats and x_sums go together: both or neither");
     const size_t dsum_bytes = fused_backward_dsum(a), need = dsum_bytes + fused_backward_parts(a);
@@ -351,11 +362,43 @@ int gridnet_hip_fused_backward(int dtype, const void *weight, const void *bias, 
     a.ln.dgamma = (float *)dgamma;
     a.ln.dbeta = (float *)dbeta;
     a.ln.x_part = x_stats ? (float *)((char *)workspace + dsum_bytes) : nullptr;
+    a.ln.residual = residual;
+    a.ln.g_prev = (const float *)g_prev;
+    a.ln.g_out = (float *)g_out;
+    a.ln.g_rows = g_out ? (const float *)g_out : (const float *)dy;
     if (int rc = step_backward_fast(a, st)) return rc;
     if (!x_stats) return GRIDNET_OK;
     const int nblk = (M / block_size) * (N / block_size) * (K / block_size);
     return layernorm_finalize_sums(a.ln.x_part, nblk * step_fast_backward_parts(block_size),
                                    (long)M * N * K, (float *)x_sums, B, st);
+}
+
+int gridnet_hip_fused_backward(int dtype, const void *weight, const void *bias, const void *scale,
+                               const void *gamma, const void *beta, const void *x,
+                               const void *x_stats, const void *dy, const void *y_raw,
+                               const void *y_stats, const void *y_sums, void *dweight, void *dbias,
+                               void *dscale, void *dgamma, void *dbeta, void *dx, void *x_sums, int B,
+                               int M, int N, int K, int inner, int block_size, int activation,
+                               int flags, void *workspace, size_t workspace_bytes, void *stream) {
+    return fused_backward(dtype, weight, bias, scale, gamma, beta, x, x_stats, dy, y_raw, y_stats,
+                          y_sums, dweight, dbias, dscale, dgamma, dbeta, dx, x_sums, B, M, N, K, inner,
+                          block_size, activation, flags, workspace, workspace_bytes, stream, 0, nullptr,
+                          nullptr);
+}
+
+int gridnet_hip_fused_backward_residual(int dtype, const void *weight, const void *bias,
+                                        const void *scale, const void *gamma, const void *beta,
+                                        const void *x, const void *x_stats, const void *dy,
+                                        const void *y_raw, const void *y_stats, const void *y_sums,
+                                        const void *g_prev, void *g_out, void *dweight, void *dbias,
+                                        void *dscale, void *dgamma, void *dbeta, void *dx,
+                                        void *x_sums, int B, int M, int N, int K, int inner,
+                                        int block_size, int activation, int flags, void *workspace,
+                                        size_t workspace_bytes, void *stream) {
+    return fused_backward(dtype, weight, bias, scale, gamma, beta, x, x_stats, dy, y_raw, y_stats,
+                          y_sums, dweight, dbias, dscale, dgamma, dbeta, dx, x_sums, B, M, N, K, inner,
+                          block_size, activation, flags, workspace, workspace_bytes, stream, 1, g_prev,
+                          g_out);
 }
 
 }  // extern "C"

@@ -24,9 +24,18 @@ struct LnFold {
     const float *y_sums;        // [B,2]: mean(g), mean(g * yhat) with g = gamma * incoming gradient
     float *dgamma, *dbeta;      // [M,N,K], summed over the batch, committed like dbias
     float *x_part;              // partial sums for the LayerNorm backward of x: [B, nblk, parts, 2]
-    // forward only: the output is x + (step(LayerNorm(x)) - LayerNorm(x)), the reference's
-    // outer_residual form (gridnet/scripts/train_imagenet.py:81-83); needs x_stats
+    // The reference's outer_residual form of the loop (gridnet/scripts/train_imagenet.py:81-83):
+    // h' = h + (step(n) - n), n = LayerNorm(h).  Forward: the output is x + (result - n); needs
+    // x_stats.  Backward of the step that produced h' from h = x, with G' the gradient with
+    // respect to h': the step's incoming gradient is G' itself, which is either given (`dy`,
+    // when y_raw is null: the last step of a chain) or formed on load as
+    // g_prev + LayerNorm'(dy; y_raw, y_stats, y_sums), the gradient with respect to h'' of the
+    // step after plus that step's dn taken through its LayerNorm, and then also stored to g_out;
+    // dx receives dn = (gradient with respect to n) - G', and x_part its LayerNorm sums.
     int residual;
+    const float *g_prev;  // [B,M,N,K] or null
+    float *g_out;         // [B,M,N,K] or null
+    const float *g_rows;  // [B,M,N,K] G' for the cross-block kernel: g_out, or dy when given
 };
 
 struct StepArgs {

@@ -792,7 +792,8 @@ __device__ __forceinline__ void commit_grads(float *base, const float (&val)[R][
     }
 }
 
-template <int BS, int CPT, int NSLOT, int ACT, bool LN>
+// RES (with LN): the outer_residual form of the loop, see LnFold.
+template <int BS, int CPT, int NSLOT, int ACT, bool LN, bool RES = false>
 __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) __attribute__((amdgpu_waves_per_eu(2)))
 void step_bwd_fast(
     const float *__restrict__ weight, const float *__restrict__ bias,
@@ -916,19 +917,24 @@ void step_bwd_fast(
     // what is requested one element ahead: the x window, the incoming gradient of the owned
     // cells and, for LN, the raw output there and the per-sample numbers of both LayerNorms
     float g[CPT], gnext[CPT], ynext[CPT], nx_mean = 0.f, nx_rstd = 1.f, ny[4] = {0.f, 1.f, 0.f, 0.f};
+    // RES: G'' of the owned cells (of the step after), G' as formed for the current element, and
+    // the latter again for the element whose results are stored one element late
+    float gprev[CPT], gin[CPT], gin_done[CPT];
+    const bool through_ln = LN && (!RES || ln.y_raw != nullptr);  // dy passes a LayerNorm on load
     auto fetch_element = [&](int s) {
         fx.fetch(x + s * cells, pre);
         load_cells<CPT>(dy + s * cells + pl.gc, gnext);
-        if (LN) {
+        if (RES && through_ln) load_cells<CPT>(ln.g_prev + s * cells + pl.gc, gprev);
+        if (through_ln) {
             load_cells<CPT>(ln.y_raw + s * cells + pl.gc, ynext);
             ny[0] = load_ahead(ln.y_stats, 2 * s);
             ny[1] = load_ahead(ln.y_stats, 2 * s + 1);
             ny[2] = load_ahead(ln.y_sums, 2 * s);
             ny[3] = load_ahead(ln.y_sums, 2 * s + 1);
-            if (ln_in) {
-                nx_mean = load_ahead(ln.x_stats, 2 * s);
-                nx_rstd = load_ahead(ln.x_stats, 2 * s + 1);
-            }
+        }
+        if (ln_in) {
+            nx_mean = load_ahead(ln.x_stats, 2 * s);
+            nx_rstd = load_ahead(ln.x_stats, 2 * s + 1);
         }
     };
     // the element just fetched becomes the current one: its gradient (through the LayerNorm
@@ -936,14 +942,16 @@ void step_bwd_fast(
     auto take_element = [&]() {
 #pragma unroll
         for (int c = 0; c < CPT; ++c) {
-            if (LN) {
+            if (through_ln) {
                 const float yh = (ynext[c] - ny[0]) * ny[1];
                 dgam[c] = fmaf(gnext[c], yh, dgam[c]);
                 dbet[c] += gnext[c];
                 g[c] = ny[1] * (gam[c] * gnext[c] - ny[2] - yh * ny[3]);
+                if (RES) g[c] += gprev[c];
             } else {
                 g[c] = gnext[c];
             }
+            if (RES) gin[c] = g[c];
         }
         if (ln_in) fx.commit_ln(win, pre, affine, nx_mean, nx_rstd);
         else fx.commit(win, pre);
@@ -967,6 +975,7 @@ void step_bwd_fast(
         store_cells<CPT>(dsum_out + o, d_done);
         if (dx_accumulate) add_cells<CPT>(dx + o, g_done);
         else store_cells<CPT>(dx + o, g_done);
+        if (RES && ln.g_out) store_cells<CPT>(ln.g_out + o, gin_done);
         done_s = -1;
     };
     for (int sb = s0; sb < s1; sb += NSLOT) {
@@ -1060,6 +1069,7 @@ void step_bwd_fast(
         for (int c = 0; c < CPT; ++c) {
             g_done[c] = g[c];
             d_done[c] = dsum[c];
+            if (RES) gin_done[c] = gin[c];
         }
         // the x windows are free (the reverse sweep does not read them): commit the next one
         if (s + NSLOT < s1) take_element();
@@ -1135,7 +1145,10 @@ void step_bwd_fast(
 // row threads, which hold the finished rows, then also form the two per-sample sums that
 // LayerNorm's backward needs, sum(gamma dx) and sum(gamma dx xhat), and leave them per 16 lanes;
 // for that they load their row of x beside their row of dx.
-template <int BS, int NSLOT, int E, bool LN>
+// RES (with LN): the outer_residual form of the loop, see LnFold: what is completed here is
+// the gradient with respect to n = LayerNorm(x), and what goes to dx (and into the sums) is
+// dn = that minus G', the gradient with respect to the step's output.
+template <int BS, int NSLOT, int E, bool LN, bool RES = false>
 __global__ __launch_bounds__((6 * BS * BS * NSLOT)) __attribute__((amdgpu_waves_per_eu(3)))
 void step_bwd_cross(
     const float *__restrict__ weight, const float *__restrict__ x, const float *__restrict__ dsum,
@@ -1223,6 +1236,7 @@ void step_bwd_cross(
     };
     float gx[E][BS];  // row threads: dx of their row so far (the own block's part)
     float xr[E][BS], xmean[E], xrstd[E];  // LN, row threads: their row of x and its statistics
+    float gr[E][BS];                       // RES, row threads: their row of G'
     int r_prev = -1;
     // the round before: its parts are all in slab `st` by now (a barrier lies in between)
     auto finish_prev = [&](int st) {
@@ -1245,6 +1259,10 @@ void step_bwd_cross(
                     load_cells<BS>(slab + (rj == 0 ? 2 : 3) * FS + ri * BS, part);
 #pragma unroll
                     for (int c = 0; c < BS; ++c) gx[e][c] += part[c];
+                }
+                if (RES) {
+#pragma unroll
+                    for (int c = 0; c < BS; ++c) gx[e][c] -= gr[e][c];
                 }
                 if (s < s1) store_cells<BS>(dx + (long)s * cells + grow, gx[e]);
                 if (ln_in) {
@@ -1279,6 +1297,7 @@ void step_bwd_cross(
             for (int e = 0; e < E; ++e) {
                 const int sc = min(sample(r, e), s1 - 1);
                 load_cells<BS>(dx + (long)sc * cells + grow, gx[e]);
+                if (RES) load_cells<BS>(ln.g_rows + (long)sc * cells + grow, gr[e]);
                 if (ln_in) {
                     load_cells<BS>(x + (long)sc * cells + grow, xr[e]);
                     xmean[e] = load_ahead(ln.x_stats, 2 * sc);
@@ -1403,12 +1422,12 @@ constexpr size_t kMaxLds = 160 * 1024;
 constexpr int kCrossSlots8 = 1, kCrossElems8 = 2;  // bs=8: 384 threads, one wave per face
 constexpr int kCrossSlots4 = 2, kCrossElems4 = 2;  // bs=4: two slots of 96 threads
 
-template <int BS, int CPT, int NSLOT, int ACT, bool LN>
+template <int BS, int CPT, int NSLOT, int ACT, bool LN, bool RES = false>
 int launch_bwd_ln(const StepArgs &a, hipStream_t st) {
     using TL = Tile<BS, CPT>;
     const long cells = (long)a.M * a.N * a.K;
     const size_t lds = bwd_lds_bytes<BS, CPT, NSLOT>(a.inner, LN);
-    auto kern = step_bwd_fast<BS, CPT, NSLOT, ACT, LN>;
+    auto kern = step_bwd_fast<BS, CPT, NSLOT, ACT, LN, RES>;
     static bool big_lds_enabled = false;            // per instantiation
     static int per_cu_cache[kMaxBackwardIters + 1];  // per instantiation, by inner iterations
     if (lds > 64 * 1024 && !big_lds_enabled) {
@@ -1455,7 +1474,7 @@ int launch_bwd_ln(const StepArgs &a, hipStream_t st) {
     // same blocks, same batch chunks; the parameter gradients are complete, dx is not yet
     constexpr int XSLOT = BS == 8 ? kCrossSlots8 : kCrossSlots4;
     constexpr int XE = BS == 8 ? kCrossElems8 : kCrossElems4;
-    hipLaunchKernelGGL((step_bwd_cross<BS, XSLOT, XE, LN>), dim3(padded_grid(p.nblk, p.nchunk)),
+    hipLaunchKernelGGL((step_bwd_cross<BS, XSLOT, XE, LN, RES>), dim3(padded_grid(p.nblk, p.nchunk)),
                        dim3(6 * BS * BS * XSLOT), 0, st, (const float *)a.weight,
                        (const float *)a.x, (const float *)a.workspace, (float *)a.dx, a.B, a.M, a.N,
                        a.K, p.nblk, p.nchunk, p.chunk_len, a.ln);
@@ -1463,6 +1482,7 @@ int launch_bwd_ln(const StepArgs &a, hipStream_t st) {
     return GRIDNET_OK;
 }
 template <int BS, int CPT, int NSLOT, int ACT> int launch_bwd(const StepArgs &a, hipStream_t st) {
+    if (a.ln.gamma && a.ln.residual) return launch_bwd_ln<BS, CPT, NSLOT, ACT, true, true>(a, st);
     if (a.ln.gamma) return launch_bwd_ln<BS, CPT, NSLOT, ACT, true>(a, st);
     return launch_bwd_ln<BS, CPT, NSLOT, ACT, false>(a, st);
 }

@@ -38,6 +38,7 @@ EXPORTS = (
     "gridnet_hip_layernorm_apply",
     "gridnet_hip_layernorm_backward_sums",
     "gridnet_hip_fused_backward",
+    "gridnet_hip_fused_backward_residual",
 )
 
 
@@ -88,6 +89,8 @@ def _load():
     lib.gridnet_hip_layernorm_backward_sums.argtypes = [i, p, p, p, p, p, i, l, p, z, p]
     lib.gridnet_hip_fused_backward.restype = i
     lib.gridnet_hip_fused_backward.argtypes = [i] + [p] * 18 + [i] * 8 + [p, z, p]
+    lib.gridnet_hip_fused_backward_residual.restype = i
+    lib.gridnet_hip_fused_backward_residual.argtypes = [i] + [p] * 20 + [i] * 8 + [p, z, p]
     return lib
 
 

@@ -11,8 +11,8 @@ loading, so the LayerNorm costs no pass over the activations of its own (one, fo
 output).  Same results within rounding; fp32, ``normalize=False``, ``inner >= 1`` only.
 
 ``outer_residual=True`` is the other shape of the loop, ``n = norm(h); h = h + (net(n) - n)``
-(gridnet/scripts/train_imagenet.py:81-83), through the fused forward entry point made for it;
-forward only (the autograd module ``GridnetBody`` trains this shape).
+(gridnet/scripts/train_imagenet.py:81-83), through the fused entry points made for it
+(``fused=True`` only).
 """
 
 import torch
@@ -58,9 +58,8 @@ class BodyRunner:
         self.on_launch = None  # optional hook(name, phase) for per-kernel timing
         self.fused = fused
         self.outer_residual = outer_residual
-        if outer_residual and (backward or not fused):
-            raise RuntimeError("outer_residual runs through the fused forward entry point only "
-                               "(fused=True, backward=False); GridnetBody trains this shape")
+        if outer_residual and not fused:
+            raise RuntimeError("outer_residual runs through the fused entry points only (fused=True)")
         if fused:
             if weight.dtype != torch.float32 or normalize or inner < 1:
                 raise RuntimeError("the fused body covers float32, normalize=False, inner >= 1")
@@ -68,6 +67,9 @@ class BodyRunner:
             self.fw_ws_bytes = _n.lib.gridnet_hip_fused_workspace_bytes(
                 batch, self.M, self.N, self.K, inner, block_size, 0)
             self.fw_ws = _n.workspace(self.fw_ws_bytes, dev)
+            if outer_residual:  # statistics of h_0 .. h_outer, and a LayerNorm output nobody reads
+                self.stats = torch.empty(keep + 1, batch, 2, device=dev, dtype=dtype)
+                self.unused = torch.empty(shape, device=dev, dtype=dtype)
             if backward:
                 self.sums = torch.empty(keep, batch, 2, device=dev, dtype=dtype)
                 self.fb_ws_bytes = _n.lib.gridnet_hip_fused_workspace_bytes(
@@ -124,14 +126,17 @@ class BodyRunner:
     def _residual_forward(self, x0):
         """h = h + (net(norm(h)) - norm(h)), ``outer`` times; returns the last h as it is."""
         stream = _n.current_stream(self.w)
+        keep = self.has_backward
+        self.x0 = x0
         # statistics of the first input: the LayerNorm entry point's, its output unused
-        self.norm_forward(x0, self.s[0], 0, stream)
+        self.norm_forward(x0, self.unused, 0, stream)
         self.stats[0, :, 0].copy_(self.mean[0])
         self.stats[0, :, 1].copy_(self.rstd[0])
         h, stats = x0, self.stats[0]
         for j in range(self.outer):
-            out = (self.s[0], self.h[1])[j % 2]
-            out_stats = self.stats[(j + 1) % 2]
+            # h[j + 1] and stats[j + 1] are kept for the backward; forward only, two of each alternate
+            out = self.h[j + 1] if keep else (self.s[0], self.h[1])[j % 2]
+            out_stats = self.stats[j + 1 if keep else (j + 1) % 2]
             self._mark("step_fwd", 0)
             _n.check(_n.lib.gridnet_hip_fused_forward_residual(
                 self.dt, self.w.data_ptr(), self.b.data_ptr(), self.r.data_ptr(),
@@ -141,6 +146,47 @@ class BodyRunner:
             self._mark("step_fwd", 1)
             h, stats = out, out_stats
         return h
+
+    def _residual_backward(self, grad_out):
+        """With G_k the gradient with respect to h_k (G_outer = grad_out): step j forms G_{j+1}
+        from G_{j+2} and the dn of step j+1 as it loads them, and leaves dn_j; the chain's input
+        gradient is G_1 + LayerNorm'(dn_0)."""
+        stream = _n.current_stream(self.w)
+        last = self.outer - 1
+        dn = [self.ga, self.gb]       # dn_j alternates between the two
+        gbuf = [self.s[0], self.s[-1]]  # G_k for 0 < k < outer: the s buffers are free in this shape
+
+        def grad_wrt(k):  # G_k
+            return grad_out if k == self.outer else gbuf[k % 2]
+
+        for j in reversed(range(self.outer)):
+            given = j == last
+            x = self.h[j] if j else self.x0
+            self._mark("step_bwd", 0)
+            _n.check(_n.lib.gridnet_hip_fused_backward_residual(
+                self.dt, self.w.data_ptr(), self.b.data_ptr(), self.r.data_ptr(),
+                self.gamma.data_ptr(), self.beta.data_ptr(), x.data_ptr(), self.stats[j].data_ptr(),
+                (grad_out if given else dn[(j + 1) % 2]).data_ptr(),
+                None if given else self.h[j + 1].data_ptr(),
+                None if given else self.stats[j + 1].data_ptr(),
+                None if given else self.sums[j + 1].data_ptr(),
+                None if given else grad_wrt(j + 2).data_ptr(),
+                None if given else grad_wrt(j + 1).data_ptr(),
+                self.dw.data_ptr(), self.db.data_ptr(), self.dr.data_ptr(), self.dgamma.data_ptr(),
+                self.dbeta.data_ptr(), dn[j % 2].data_ptr(), self.sums[j].data_ptr(),
+                self.B, self.M, self.N, self.K, self.inner, self.bs, self.act,
+                _n.OVERWRITE_PARAMS if given else 0, self.fb_ws.data_ptr(), self.fb_ws_bytes, stream))
+            self._mark("step_bwd", 1)
+        # the LayerNorm in front of the first step: dx0 = G_1 + LayerNorm'(dn_0), with its dgamma, dbeta
+        self._mark("ln_bwd", 0)
+        _n.check(_n.lib.gridnet_hip_layernorm_backward(
+            self.dt, dn[0].data_ptr(), self.x0.data_ptr(), self.gamma.data_ptr(),
+            self.mean[0].data_ptr(), self.rstd[0].data_ptr(), dn[1].data_ptr(),
+            self.dgamma.data_ptr(), self.dbeta.data_ptr(), self.B, self.n, 0,
+            self.ln_ws.data_ptr(), self.ln_ws_bytes, stream))
+        self._mark("ln_bwd", 1)
+        torch.add(dn[1], grad_wrt(1), out=dn[1])
+        return self.dw, self.db, self.dr, self.dgamma, self.dbeta, dn[1]
 
     def _fused_backward(self, grad_out):
         stream = _n.current_stream(self.w)
@@ -192,6 +238,8 @@ class BodyRunner:
         """Backward of the last ``forward``.  Returns (dweight, dbias, dscale, dgamma, dbeta, dx0);
         parameter gradients are summed over the outer steps (shared parameters)."""
         assert self.has_backward
+        if self.outer_residual:
+            return self._residual_backward(grad_out)
         if self.fused:
             return self._fused_backward(grad_out)
         stream = _n.current_stream(self.w)

@@ -158,7 +158,7 @@ int gridnet_hip_fused_forward(int dtype, const void *weight, const void *bias, c
                               int K, int inner, int block_size, double ln_eps, int activation,
                               void *workspace, size_t workspace_bytes, void *stream);
 
-/* The reference's outer_residual form of one outer step, forward only
+/* The reference's outer_residual form of one outer step, forward
  * (gridnet/scripts/train_imagenet.py:81-83: n = norm(h); h = h + (net(n) - n)):
  * y = x + (step(n) - n) with n = LayerNorm(x; x_stats, gamma, beta), y_stats = statistics of y,
  * which the next step of such a chain takes as its x_stats.  x_stats is required (the
@@ -195,6 +195,30 @@ int gridnet_hip_fused_backward(int dtype, const void *weight, const void *bias, 
                                void *dscale, void *dgamma, void *dbeta, void *dx, void *x_sums, int B,
                                int M, int N, int K, int inner, int block_size, int activation,
                                int flags, void *workspace, size_t workspace_bytes, void *stream);
+
+/* Backward of gridnet_hip_fused_forward_residual for the step that made h' = y from h = x.
+ * With G' the gradient with respect to h':
+ *   - the last step of a chain is given it: dy = G', and y_raw, y_stats, y_sums, g_prev, g_out
+ *     are all NULL;
+ *   - any other step forms it while loading: G' = g_prev + LayerNorm'(dy), where dy is the dx
+ *     that the call for the step AFTER this one wrote, y_raw = h' (that step's input),
+ *     y_stats / y_sums its statistics and the x_sums of that call, and g_prev the G'' of that
+ *     call (its g_out, or its dy if it was the last step); G' is also stored to g_out.
+ * dx receives dn = (gradient with respect to LayerNorm(x)) - G' and x_sums its LayerNorm sums;
+ * dgamma, dbeta receive the gradients of the LayerNorm that dy was taken through.  What remains
+ * for the caller after the first step of the chain (x = the chain's input): the gradient of that
+ * input is G' + LayerNorm'(dx), with the LayerNorm's dgamma, dbeta on top: one
+ * gridnet_hip_layernorm_backward call and an addition.  Flags, workspace and everything else as
+ * gridnet_hip_fused_backward. */
+int gridnet_hip_fused_backward_residual(int dtype, const void *weight, const void *bias,
+                                        const void *scale, const void *gamma, const void *beta,
+                                        const void *x, const void *x_stats, const void *dy,
+                                        const void *y_raw, const void *y_stats, const void *y_sums,
+                                        const void *g_prev, void *g_out, void *dweight, void *dbias,
+                                        void *dscale, void *dgamma, void *dbeta, void *dx,
+                                        void *x_sums, int B, int M, int N, int K, int inner,
+                                        int block_size, int activation, int flags, void *workspace,
+                                        size_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

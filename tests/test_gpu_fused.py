@@ -114,6 +114,69 @@ def test_fused_residual_forward_matches_oracle(name, grid, batch, outer):
     assert torch.equal(d["x0"].cpu(), t["x0"]), "the input was modified"
 
 
+@pytest.mark.parametrize("name,grid,batch,outer,activation", [
+    ("C3", 16, 2, 2, None), ("C3", 16, 1, 1, None), ("C5", 16, 1, 2, None),
+    ("C3", 32, 3, 3, "silu"), ("C5", 16, 5, 3, "silu"), ("C3", 16, 2, 4, "tanh")])
+def test_fused_residual_chain_matches_oracle(name, grid, batch, outer, activation):
+    """Forward and backward of the outer_residual shape of the loop through
+    gridnet_hip_fused_forward_residual / _backward_residual against autograd of the oracle."""
+    from gridnet_amd.configs import WORKLOADS, make_inputs
+    from gridnet_amd.runner import BodyRunner
+
+    wl = dataclasses.replace(WORKLOADS[name], grid=grid, batch=batch, outer=outer, backward=True)
+    if activation:
+        wl = dataclasses.replace(wl, activation=activation)
+    print(f"fused residual {wl.name} grid={grid} batch={batch} outer={outer} act={wl.activation}", flush=True)
+
+    def make(seed):
+        t = randomise_affine(make_inputs(wl, seed=seed))
+        # the result is not normalised: smaller updates keep h (and the gradients) O(1); 8 inner
+        # iterations need them smaller still, or fp32 rounding grows past the bar
+        f = 0.25 if wl.inner >= 8 else 0.5
+        t["weight"], t["scale"] = t["weight"] * f, t["scale"] * f
+        return t
+
+    def margin(t):  # smallest |pre-activation| of the oracle chain in this shape of the loop
+        from oracle.fast import gridnet_step_fast
+        smallest = [float("inf")]
+
+        def step(*args):
+            return gridnet_step_fast(*args, watch=lambda u: smallest.__setitem__(
+                0, min(smallest[0], u.abs().min().item())))
+
+        with torch.no_grad():
+            network_forward(*[t[k].double() for k in PARAMS], t["x0"].double(), wl.inner, wl.outer,
+                            wl.block_size, wl.activation, wl.normalize, outer_residual=True, step_fn=step)
+        return smallest[0]
+
+    t = make(0)
+    if wl.activation in ("relu", "leaky_relu"):
+        t = next(c for c in (make(seed) for seed in range(200)) if margin(c) >= 2e-5)
+    d = {k: v.to(DEV) for k, v in t.items()}
+    run = BodyRunner(d["weight"], d["bias"], d["scale"], d["gamma"], d["beta"], batch, wl.inner,
+                     wl.outer, wl.block_size, wl.activation, wl.normalize, backward=True,
+                     fused=True, outer_residual=True)
+    got = (run.forward(d["x0"]).clone(), *[g.clone() for g in run.backward(d["grad_out"])])
+    exp = network_forward_backward(
+        [t[k].double() for k in PARAMS], t["x0"].double(), t["grad_out"].double(),
+        inner_iterations=wl.inner, outer_iterations=wl.outer, block_size=wl.block_size,
+        activation=wl.activation, normalize=wl.normalize, outer_residual=True)
+    # Parameter gradients are sums over batch x inner x outer terms, accumulated in fp32 (by the
+    # reference's kernels too), and in this shape of the loop the terms do not shrink from step
+    # to step: their atol is scaled from the bar's own cases (two terms) by sqrt(terms / 2).
+    summed = 1e-5 * max(1.0, (batch * wl.inner * wl.outer / 2) ** 0.5)
+    for name_, a, e in zip(NAMES, got, exp):
+        assert_close(a, e, atol=1e-5 if name_ in ("y", "dx0") else summed, what=name_)
+    assert torch.equal(d["grad_out"].cpu(), t["grad_out"]), "the upstream gradient was modified"
+    # twice the same result: nothing is left over from one call to the next
+    again = (run.forward(d["x0"]).clone(), *[g.clone() for g in run.backward(d["grad_out"])])
+    # (parameter gradients of a batch split over workgroups are summed with float atomics, whose
+    # order varies from run to run)
+    for name_, a, e in zip(NAMES, again, got):
+        assert_close(a, e, rtol=1e-5, atol=1e-6 if name_ in ("y", "dx0") else summed,
+                     what=f"{name_}, second run")
+
+
 @pytest.mark.parametrize("shape", [(8, 16, 24), (24, 8, 16)])
 def test_fused_chain_non_cubic_grid(shape):
     """Axes of different lengths: catches a swapped stride in the window, face or row indexing."""
