@@ -18,6 +18,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor peak
+FP32_PEAK_TFLOPS = 157.3  # MI355X vector fp32, vendor peak (with packed fp32 instructions)
 
 
 def gpu_run(wl, steps, warmup, fused, graph_replay=True):
@@ -181,6 +182,11 @@ def main():
         pass
     dom_s = kernel_s[dominant]
     achieved = bytes_[dominant] / dom_s / 1e9
+    # the same entry point against the vector ALU: algorithmic fp32 FMAs per cell-update (27 for
+    # the update itself; 81 in the backward: recompute, weight gradient, input gradient)
+    fma = {"step_fwd": 27, "step_bwd": 81}.get(dominant)
+    per_launch = wl.cell_updates / wl.outer
+    tflops = None if fma is None else 2 * fma * per_launch / dom_s / 1e12
     out = {
         "metric": "cell-updates/s fwd+bwd, 64^3 grid 8^3 blocks batch 32; % of HBM roofline",
         "value": wl.cell_updates / wall,
@@ -211,6 +217,11 @@ def main():
             "frac": achieved / HBM_PEAK_GBS,
             "traffic": traffic,
         },
+        # informational: this build compiles with packed fp32 arithmetic switched off, which
+        # halves the vector fp32 peak it can reach
+        "vector_alu": {"kernel": dominant, "achieved": tflops, "unit": "TFLOP/s",
+                       "peak": FP32_PEAK_TFLOPS, "peak_without_packed_fp32": FP32_PEAK_TFLOPS / 2,
+                       "frac": None if tflops is None else tflops / FP32_PEAK_TFLOPS},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(wl)
