@@ -11,6 +11,9 @@
  *     t = 9a + 3b + c addressing neighbour (i+a-1, j+b-1, k+c-1); bias, scale [M, N, K];
  *     activations [B, M, N, K].  (gridnet/__init__.py:42-49, gridnet/backend_torch.py:283-298)
  *   - `dtype` is GRIDNET_F32 or GRIDNET_F64 and applies to every tensor of the call.
+ *   - A tensor may start at any address that is a multiple of its element size (for example
+ *     a view one element into a larger buffer), as with the reference's element-wise
+ *     accessors (src/gridnet_cuda_kernels.cu:103-107); the workspace likewise.
  *   - Return value 0 = enqueued.  Non-zero = nothing was enqueued; the message is
  *     available from gridnet_hip_last_error() on the calling thread.
  */
