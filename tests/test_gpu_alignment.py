@@ -112,6 +112,11 @@ def test_fused_chain_with_tensors_at_odd_addresses():
     def call(place):
         run = BodyRunner(*(place(t.to(DEV)) for t in (w, b, r, gamma, beta)), batch, inner, outer, bs,
                          "silu", backward=True, fused=True)
+        if place is odd:  # the workspaces too: four bytes past the allocator's alignment
+            for name in ("fw_ws", "fb_ws", "ln_ws", "bw_ws"):
+                nbytes = getattr(run, name).numel()
+                setattr(run, name, torch.empty(nbytes + 4, dtype=torch.uint8, device=DEV)[4:])
+                assert getattr(run, name).data_ptr() % 8 == 4
         y = run.forward(place(x.to(DEV)))
         grads = run.backward(place(gy.to(DEV)))
         torch.cuda.synchronize()
