@@ -172,6 +172,7 @@ __global__ __launch_bounds__(BS *BS *BS) void step_bwd_generic(
         for (int idx = tid; idx < G::W; idx += G::NT) gwin[idx] = T(0);
         __syncthreads();
         gwin[centre] = dy[s * cells + gc];
+        if (inner == 0) __syncthreads();  // no loop barrier lies before the window is read below
 
         // forward recompute, remembering this cell's trajectory
         T cur = win[centre];

@@ -71,6 +71,9 @@ MATRIX = [
     ((8, 16, 8), 4, 3, False, "relu"),
     ((8, 16, 8), 8, 5, True, "tanh"),
     ((8, 16, 8), 4, 3, True, "relu"),
+    # no inner iteration on a grid of several blocks: the gradient passes through unchanged
+    ((16, 24, 16), 8, 0, True, "silu"),
+    ((8, 16, 8), 4, 0, False, "tanh"),
 ]
 
 
@@ -79,7 +82,7 @@ def test_step_parity_fp32(case):
     compare(case)
 
 
-@pytest.mark.parametrize("case", MATRIX[:6] + MATRIX[9:11],
+@pytest.mark.parametrize("case", MATRIX[:6] + MATRIX[9:11] + MATRIX[-2:],
                          ids=lambda c: "-".join(map(str, c)).replace(" ", ""))
 def test_step_parity_fp64(case):
     compare(case, dtype=torch.float64, rtol=1e-9, atol=1e-9)

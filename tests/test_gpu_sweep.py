@@ -1,0 +1,119 @@
+"""Seeded random sweep over shapes the hand-picked cases leave out.
+
+The tuned fp32 kernels choose their launch plan from the shape (batch chunks per workgroup,
+slots per workgroup, whether a workgroup owns the whole batch of its block, atomics or plain
+stores for the parameter gradients), so a fixed list of cases exercises a fixed set of plans.
+Here grid, block size, batch, inner iterations, activation and the accumulate/overwrite flags are
+drawn at random (fixed seeds) and every draw is held to the generic kernels run in fp64 on the
+same fp32 inputs -- the two share no device code, and each is held to the CPU oracle elsewhere
+(test_gpu_step.py).  A second sweep holds the chain with the LayerNorm folded into the step
+kernels to the op-by-op chain of the same library, in both shapes of the loop."""
+
+import math
+import random
+
+import pytest
+import torch
+
+from helpers import assert_close, make_acts, make_params
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+SMOOTH = ("silu", "tanh")  # gradients under relu/leaky_relu flip at the kink in fp32 vs fp64
+
+
+def draw_step(seed):
+    rng = random.Random(seed)
+    bs = rng.choice((4, 8))
+    dims = tuple(bs * rng.randint(1, 5 if bs == 4 else 3) for _ in range(3))
+    batch = rng.choice((1, 2, 3, 5, 8, 13, 31, 32, 33, 47, 64, 70))
+    inner = rng.choice((0, 1, 1, 2, 3, 4, 5, 7))
+    return dims, bs, batch, inner, rng.choice(SMOOTH), rng.random() < 0.5
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_step_tuned_fp32_against_generic_fp64(seed):
+    import gridnet_cuda
+
+    shape, bs, batch, inner, activation, preset = draw_step(seed)
+    print(f"sweep step seed={seed} shape={shape} bs={bs} B={batch} inner={inner} act={activation} "
+          f"preset={preset}", flush=True)
+    w, b, r = make_params(shape, seed=1000 + seed)
+    if inner >= 5:
+        w, r = w * 0.5, r * 0.5
+    x, gy = make_acts(batch, shape, seed=2000 + seed), make_acts(batch, shape, seed=3000 + seed)
+    # gradient buffers arrive holding something (the entry point accumulates), or zero-filled
+    start = [make_acts(1, t.shape, seed=4000 + seed + i)[0] if preset else torch.zeros_like(t)
+             for i, t in enumerate((w, b, r, x))]
+
+    def call(dtype):
+        tw, tb, tr, tx, tgy = (t.to(device=DEV, dtype=dtype) for t in (w, b, r, x, gy))
+        y = torch.full_like(tx, float("nan"))
+        gridnet_cuda.forward(tw, tb, tr, tx, y, inner, bs, 1e-5, False, activation)
+        outs = [t.to(device=DEV, dtype=dtype) for t in start]
+        gridnet_cuda.backward(tw, tb, tr, tx, tgy, *outs, inner, bs, 1e-5, False, activation)
+        return [y] + outs
+
+    fast, slow = call(torch.float32), call(torch.float64)
+    summed = 1e-5 * max(1.0, math.sqrt(batch * max(inner, 1) / 2))
+    for name, got, want in zip(("y", "dweight", "dbias", "dscale", "dx"), fast, slow):
+        assert torch.isfinite(got).all(), name
+        assert_close(got, want, atol=summed if name in ("dweight", "dbias", "dscale") else 1e-5,
+                     what=name)
+
+
+def draw_chain(seed):
+    rng = random.Random(100 + seed)
+    bs = rng.choice((4, 8))
+    dims = tuple(bs * rng.randint(1, 4 if bs == 4 else 2) for _ in range(3))
+    batch = rng.choice((1, 2, 5, 9, 32, 40))
+    inner = rng.choice((1, 2, 3, 4))
+    outer = rng.choice((1, 2, 3, 5))
+    return dims, bs, batch, inner, outer, rng.choice(SMOOTH + ("leaky_relu",)), rng.random() < 0.4
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_chain_fused_against_op_by_op(seed):
+    from gridnet_amd.network import GridnetBody
+    from gridnet_amd.runner import BodyRunner
+
+    shape, bs, batch, inner, outer, activation, residual = draw_chain(seed)
+    print(f"sweep chain seed={seed} shape={shape} bs={bs} B={batch} inner={inner} outer={outer} "
+          f"act={activation} residual={residual}", flush=True)
+    w, b, r = make_params(shape, seed=5000 + seed)
+    w = w * 0.5
+    gamma = 1 + 0.2 * make_acts(1, shape, seed=5100 + seed)[0]
+    beta = 0.2 * make_acts(1, shape, seed=5200 + seed)[0]
+    x, gy = make_acts(batch, shape, seed=5300 + seed), make_acts(batch, shape, seed=5400 + seed)
+    params = [t.to(DEV) for t in (w, b, r, gamma, beta)]
+
+    run = BodyRunner(*params, batch, inner, outer, bs, activation, backward=True, fused=True,
+                     outer_residual=residual)
+    y = run.forward(x.to(DEV)).clone()
+    fused = [y] + [g.clone() for g in run.backward(gy.to(DEV))]
+
+    # the same chain op by op through the autograd wrappers (one call per step and LayerNorm)
+    body = GridnetBody(shape, inner, outer, bs, activation=activation, outer_residual=residual,
+                       device=DEV)
+    with torch.no_grad():
+        for p, t in zip((body.network.weight, body.network.bias, body.network.residual_scale, body.norm.weight,
+                         body.norm.bias), params):
+            p.copy_(t)
+    x0 = x.to(DEV).requires_grad_(True)
+    out = body(x0)
+    leaves = [body.network.weight, body.network.bias, body.network.residual_scale, body.norm.weight,
+              body.norm.bias, x0]
+    grads = torch.autograd.grad(out, leaves, gy.to(DEV))
+    steps = [out.detach()] + list(grads)
+
+    terms = batch * inner * outer
+    summed = 1e-5 * max(1.0, math.sqrt(terms / 2))
+    names = ("y", "dweight", "dbias", "dscale", "dgamma", "dbeta", "dx0")
+    if activation == "leaky_relu":
+        # both chains are fp32, but they round differently: a pre-activation within rounding
+        # distance of the kink can take different branches.  The forward result is continuous.
+        names, fused, steps = names[:1], fused[:1], steps[:1]
+    for name, got, want in zip(names, fused, steps):
+        assert torch.isfinite(got).all(), name
+        assert_close(got, want, atol=summed if name.startswith("d") and name != "dx0" else 1e-5,
+                     what=name)
