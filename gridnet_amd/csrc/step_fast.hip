@@ -264,6 +264,34 @@ template <typename TL, int NT = TL::TPS> struct Fetch {  // NT: threads of a slo
                 }
             }
     }
+    // The plain commit, which also adds up what it writes: (sum, sum of squares) of the halo
+    // entries in part[0..1], of the block's own cells in part[2..3] (entries outside the grid are
+    // zeros and add nothing).  For the per-window normalisation.
+    template <int COPIES = 2>
+    __device__ __forceinline__ void commit_sums(float *win, const Buf &v, float (&part)[4]) const {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) part[q] = 0.f;
+#pragma unroll
+        for (int e = 0; e < RPT; ++e)
+            if (loff[e] >= 0) {
+                const int row = (lane0 + e * NT) >> 1;
+                const int wj = row % S, wi = row / S;
+                const bool halo_row = wi == 0 || wi == S - 1 || wj == 0 || wj == S - 1;
+                const float end = (ok[e] && edge_ok[e]) ? v[e][HC] : 0.f;
+                float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+                for (int q = 0; q < HC; ++q) {
+                    const float c = ok[e] ? v[e][q] : 0.f;
+                    s1 += c;
+                    s2 = fmaf(c, c, s2);
+                }
+                part[0] += end + (halo_row ? s1 : 0.f);
+                part[1] += fmaf(end, end, halo_row ? s2 : 0.f);
+                part[2] += halo_row ? 0.f : s1;
+                part[3] += halo_row ? 0.f : s2;
+            }
+        commit<COPIES>(win, v);
+    }
     // The same, with the LayerNorm of the producer applied on the way in: an entry becomes
     // (v - mean) * rstd * gamma + beta; entries outside the grid stay zero.  gamma and beta of a
     // thread's half rows sit in LDS packed per half row, [gamma cells | beta cells | gamma end,
@@ -434,15 +462,28 @@ constexpr int kFwdDepth = 9;  // neighbour rows requested ahead of the arithmeti
 // RES (with LN): the output is x + (result - LayerNorm(x)), the reference's outer_residual form
 // (gridnet/scripts/train_imagenet.py:81-83); the statistics left for the next LayerNorm are
 // those of that output.
-template <int BS, int CPT, int NSLOT, int ACT, bool LN, bool RES = false>
+// NORM: per-window normalisation (gridnet/backend_torch.py:126-129,
+// src/gridnet_cuda_kernels.cu:164-170): before every inner iteration the whole (bs+2)^3 window,
+// halo and zeros outside the grid included, is brought to mean 0 and divided by (std + eps); the
+// stencil reads the normalised values, the residual adds to the raw ones.  With S = sum_t w_t x_t
+// over the RAW window the pre-activation is b + (S - mean * sum_t w_t) / (std + eps), so the
+// stencil itself is unchanged; the statistics come from sums the threads keep of their own
+// cells (the halo never changes, its sums are taken once, when the window is committed).
+template <int BS, int CPT, int NSLOT, int ACT, bool LN, bool RES = false, bool NORM = false>
 __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) __attribute__((amdgpu_waves_per_eu(3)))
 void step_fwd_fast(
     const float *__restrict__ weight, const float *__restrict__ bias,
     const float *__restrict__ scale, const float *__restrict__ x, float *__restrict__ y, int B, int M,
-    int N, int K, int inner, int nblk, int nchunk, int chunk_len, LnFold ln) {
+    int N, int K, int inner, int nblk, int nchunk, int chunk_len, LnFold ln, float norm_eps) {
     using TL = Tile<BS, CPT>;
-    // per slot two copies of the window; then, for the folded LayerNorm, the packed gamma/beta
-    __shared__ __attribute__((aligned(16))) float lds[NSLOT * 2 * TL::WIN + (LN ? Fetch<TL>::AFFINE : 0)];
+    constexpr int GROUPS = TL::TPS / 16;  // 16-lane groups of a slot
+    constexpr int NORM_FLOATS = NORM ? NSLOT * GROUPS * (4 + 2 * 2) : 0;
+    // per slot two copies of the window; then, for the folded LayerNorm, the packed gamma/beta;
+    // then, for NORM, per slot and 16-lane group the sums taken at commit and, twice (alternating
+    // between inner iterations), the sums of the owned cells
+    __shared__ __attribute__((aligned(16))) float
+        lds[NSLOT * 2 * TL::WIN + (LN ? Fetch<TL>::AFFINE : 0) + NORM_FLOATS];
+    static_assert(!(NORM && (LN || RES)), "the folded LayerNorm comes without normalisation");
 
     int blk, chunk;
     if (!split_block_id(blockIdx.x, nblk, nchunk, blk, chunk)) return;  // grid padding
@@ -458,6 +499,21 @@ void step_fwd_fast(
     for (int t = 0; t < 27; ++t) load_cells<CPT>(weight + t * cells + pl.gc, w[t]);
     load_cells<CPT>(bias + pl.gc, bv);
     load_cells<CPT>(scale + pl.gc, rv);
+    // NORM: sum of the 27 weights of every owned cell; the sums of this slot in LDS
+    float wsum[CPT], zero[CPT];
+    float *sums_at_commit = lds + NSLOT * 2 * TL::WIN + (LN ? Fetch<TL>::AFFINE : 0) + pl.slot * GROUPS * 8;
+    float *own_sums = sums_at_commit + GROUPS * 4;  // [2][GROUPS][2]
+    const int group = pl.lane / 16;
+    constexpr float inv_count = 1.f / (TL::S * TL::S * TL::S);
+    if (NORM) {
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) {
+            zero[c] = 0.f;
+            wsum[c] = 0.f;
+#pragma unroll
+            for (int t = 0; t < 27; ++t) wsum[c] += w[t][c];
+        }
+    }
     typename Fetch<TL>::Buf pre;
     if (ln_in) {  // gamma and beta of the window, once per workgroup
         if (pl.slot == 0) {
@@ -490,12 +546,21 @@ void step_fwd_fast(
         const bool active = s < s1;  // a slot past the end idles through the barriers
         if (active) {
             if (ln_in) fx.commit_ln(win, pre, affine, pre_mean, pre_rstd);
-            else fx.commit(win, pre);
+            else if (NORM) {
+                float part[4];
+                fx.commit_sums(win, pre, part);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) part[q] = row16_sum(part[q]);
+                if ((pl.lane & 15) == 0)
+                    *reinterpret_cast<float4 *>(sums_at_commit + group * 4) =
+                        make_float4(part[0], part[1], part[2], part[3]);
+            } else fx.commit(win, pre);
         }
         lds_barrier();
         if (done_s >= 0) store_cells<CPT>(y + done_s * cells + pl.gc, done);
         if (s + NSLOT < s1) fetch_element(s + NSLOT);  // next element, in flight
         float cur[CPT], base[CPT], raw[CPT];
+        float halo1 = 0.f, halo2 = 0.f, own1 = 0.f, own2 = 0.f;  // NORM: sums of the window
         if (active) {
 #pragma unroll
             for (int c = 0; c < CPT; ++c) cur[c] = win[pl.own + c];
@@ -504,15 +569,50 @@ void step_fwd_fast(
 #pragma unroll
                 for (int c = 0; c < CPT; ++c) base[c] = cur[c];
             }
+            if (NORM) {
+#pragma unroll
+                for (int q = 0; q < GROUPS; ++q) {  // fixed order: every thread gets the same sums
+                    const float4 p4 = *reinterpret_cast<const float4 *>(sums_at_commit + q * 4);
+                    halo1 += p4.x; halo2 += p4.y; own1 += p4.z; own2 += p4.w;
+                }
+            }
         }
         for (int it = 0; it < inner; ++it) {
             if (active) {
                 float u[CPT];
-                stencil<TL, CPT, kFwdDepth>(win + (it & 1) * TL::WIN, pl.row00, w, bv, u);
+                if (NORM) {
+                    if (it > 0) {
+                        own1 = own2 = 0.f;
+#pragma unroll
+                        for (int q = 0; q < GROUPS; ++q) {
+                            const float2 p2 = *reinterpret_cast<const float2 *>(
+                                own_sums + ((it & 1) * GROUPS + q) * 2);
+                            own1 += p2.x; own2 += p2.y;
+                        }
+                    }
+                    const float mean = (halo1 + own1) * inv_count;
+                    const float var = fmaxf(fmaf(-mean, mean, (halo2 + own2) * inv_count), 0.f);
+                    const float inv = 1.f / (sqrtf(var) + norm_eps);
+                    stencil<TL, CPT, kFwdDepth>(win + (it & 1) * TL::WIN, pl.row00, w, zero, u);
+#pragma unroll
+                    for (int c = 0; c < CPT; ++c) u[c] = fmaf(inv, fmaf(-mean, wsum[c], u[c]), bv[c]);
+                } else {
+                    stencil<TL, CPT, kFwdDepth>(win + (it & 1) * TL::WIN, pl.row00, w, bv, u);
+                }
+                float s1 = 0.f, s2 = 0.f;
 #pragma unroll
                 for (int c = 0; c < CPT; ++c) {
                     cur[c] = fmaf(rv[c], Act<ACT, float>::f(u[c]), cur[c]);
                     win[((it + 1) & 1) * TL::WIN + pl.own + c] = cur[c];
+                    s1 += cur[c];
+                    s2 = fmaf(cur[c], cur[c], s2);
+                }
+                if (NORM && it + 1 < inner) {  // the owned cells' part of the next statistics
+                    s1 = row16_sum(s1);
+                    s2 = row16_sum(s2);
+                    if ((pl.lane & 15) == 0)
+                        *reinterpret_cast<float2 *>(own_sums + (((it + 1) & 1) * GROUPS + group) * 2) =
+                            make_float2(s1, s2);
                 }
             }
             lds_barrier();
@@ -1386,10 +1486,10 @@ Plan make_plan(const StepArgs &a, int nslot, int resident, bool whole_batch_per_
     return p;
 }
 
-template <int BS, int CPT, int NSLOT, int ACT, bool LN, bool RES = false>
+template <int BS, int CPT, int NSLOT, int ACT, bool LN, bool RES = false, bool NORM = false>
 int launch_fwd_ln(const StepArgs &a, hipStream_t st) {
     using TL = Tile<BS, CPT>;
-    auto kern = step_fwd_fast<BS, CPT, NSLOT, ACT, LN, RES>;
+    auto kern = step_fwd_fast<BS, CPT, NSLOT, ACT, LN, RES, NORM>;
     static int per_cu = 0;
     if (per_cu == 0) {
         int n = 0;
@@ -1402,7 +1502,7 @@ int launch_fwd_ln(const StepArgs &a, hipStream_t st) {
     hipLaunchKernelGGL(kern, dim3(padded_grid(p.nblk, p.nchunk)), dim3(TL::TPS * NSLOT), 0, st,
                        (const float *)a.weight, (const float *)a.bias, (const float *)a.scale,
                        (const float *)a.x, (float *)a.y, a.B, a.M, a.N, a.K, a.inner, p.nblk, p.nchunk,
-                       p.chunk_len, a.ln);
+                       p.chunk_len, a.ln, (float)a.eps);
     return check_launch("step_fwd_fast");
 }
 template <int ACT, bool LN, bool RES = false> int launch_fwd_split(const StepArgs &a, hipStream_t st) {
@@ -1421,6 +1521,7 @@ template <int ACT, bool LN, bool RES = false> int launch_fwd_split(const StepArg
     return check_launch("step_fwd_split");
 }
 template <int BS, int CPT, int NSLOT, int ACT> int launch_fwd(const StepArgs &a, hipStream_t st) {
+    if (a.normalize) return launch_fwd_ln<BS, CPT, NSLOT, ACT, false, false, true>(a, st);
     if (a.ln.gamma && a.ln.residual) {
         if (BS == 8) return launch_fwd_split<ACT, true, true>(a, st);
         return launch_fwd_ln<BS, CPT, NSLOT, ACT, true, true>(a, st);
@@ -1535,7 +1636,8 @@ int step_fast_forward_part_count(int block_size) { return 16 * (block_size == 8 
 int step_fast_backward_parts(int block_size) { return block_size * block_size / 16; }
 
 bool step_fast_supports(const StepArgs &a, bool backward) {
-    if (a.dtype != GRIDNET_F32 || a.normalize) return false;
+    if (a.dtype != GRIDNET_F32) return false;
+    if (a.normalize && (backward || a.ln.gamma)) return false;  // forward only, plain step only
     if (a.block_size != 4 && a.block_size != 8) return false;
     if (backward) {
         const bool ln = a.ln.gamma != nullptr;
