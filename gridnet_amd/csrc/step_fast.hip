@@ -89,6 +89,21 @@ __device__ __forceinline__ float row16_sum(float v) {
     return v;
 }
 
+// Sum of `v` over those lanes of the calling wave that belong to the caller's slot: the whole
+// wave for slots of 64 threads and more, the caller's half of it for 32-thread slots.  Row
+// rotations, then the four row totals are read across as scalars: no LDS, and every lane of the
+// slot gets the same bits.
+template <int TPS> __device__ __forceinline__ float slot_wave_sum(float v) {
+    static_assert(TPS == 32 || TPS % 64 == 0, "slots are half waves or whole waves");
+    const int r = __float_as_int(row16_sum(v));
+    const float r0 = __int_as_float(__builtin_amdgcn_readlane(r, 0));
+    const float r1 = __int_as_float(__builtin_amdgcn_readlane(r, 16));
+    const float r2 = __int_as_float(__builtin_amdgcn_readlane(r, 32));
+    const float r3 = __int_as_float(__builtin_amdgcn_readlane(r, 48));
+    if (TPS == 32) return (threadIdx.x & 32) ? r2 + r3 : r0 + r1;
+    return (r0 + r1) + (r2 + r3);
+}
+
 // Load p[i], i the same for the whole wave, as a VECTOR memory load.  Left alone the compiler
 // makes it a scalar load; those return out of order and share their counter with LDS, so one
 // that is still on its way stalls the next LDS access for a whole trip to memory -- and the
@@ -874,10 +889,21 @@ constexpr int kBwdDepth = 4;  // neighbour rows requested ahead of the arithmeti
 template <int BS, int CPT> __host__ __device__ constexpr int bwd_slot_floats(int inner) {
     return 4 * Tile<BS, CPT>::WIN + inner * Tile<BS, CPT>::TPS * 2 * CPT;
 }
+// NORM, per slot behind all of the above: (mean, std, 1/(std+eps), -) of the window before
+// every inner iteration, then the sums the waves of a slot exchange: 4 floats per wave taken
+// at commit, 2 x 2 per wave for the owned cells (alternating between iterations), 2 per wave in
+// the reverse sweep
+template <int BS, int CPT> __host__ __device__ constexpr int bwd_norm_waves() {
+    return Tile<BS, CPT>::TPS >= 64 ? Tile<BS, CPT>::TPS / 64 : 1;
+}
+template <int BS, int CPT> __host__ __device__ constexpr int bwd_norm_floats(int inner) {
+    return 4 * inner + 12 * bwd_norm_waves<BS, CPT>();
+}
 // ... and at least the 27 weight planes of the block, which pass through LDS once at set-up
-template <int BS, int CPT, int NSLOT> size_t bwd_lds_bytes(int inner, bool ln = false) {
+template <int BS, int CPT, int NSLOT> size_t bwd_lds_bytes(int inner, bool ln = false, bool norm = false) {
     const size_t run = ((size_t)NSLOT * bwd_slot_floats<BS, CPT>(inner) +
-                        (ln ? Fetch<Tile<BS, CPT>>::AFFINE : 0)) * sizeof(float);
+                        (ln ? Fetch<Tile<BS, CPT>>::AFFINE : 0) +
+                        (norm ? NSLOT * bwd_norm_floats<BS, CPT>(inner) : 0)) * sizeof(float);
     const size_t setup = (size_t)27 * BS * BS * BS * sizeof(float);
     return run > setup ? run : setup;
 }
@@ -906,15 +932,35 @@ __device__ __forceinline__ void commit_grads(float *base, const float (&val)[R][
 }
 
 // RES (with LN): the outer_residual form of the loop, see LnFold.
-template <int BS, int CPT, int NSLOT, int ACT, bool LN, bool RES = false>
+// NORM: per-window normalisation (see step_fwd_fast).  With mean_i, std_i, inv_i = 1/(std_i+eps)
+// of the window before iteration i, n_i = (x_i - mean_i) inv_i what the stencil reads, and
+// dn_i[k] = sum of w_t[c] delta_i[c] over the (c, t) that read window entry k, the gradient that
+// iteration i adds to window entry k is (N = (bs+2)^3 entries)
+//   inv_i (dn_i[k] - A_i / N) - (x_i[k] - mean_i) C_i,   A_i = sum_k dn_i[k],
+//   C_i = inv_i^2 / (N std_i) * sum_k dn_i[k] (x_i[k] - mean_i).
+// Both sums run over the whole window.  The owned cells' part comes from the gather of the
+// reverse sweep; the halo's part needs no halo entry of dn: summed over the halo,
+// dn_i = sum_c delta_i[c] * (sum of c's weights whose taps read the halo) and
+// dn_i x = sum_c delta_i[c] * (those weights times the halo values they read), and both
+// brackets are fixed for the element (the halo is frozen).  What the HALO entries receive over
+// all iterations is, for halo entry h,
+//   sum over (c, t) reading h of w_t[c] D1[c]  -  x_h Q + R,
+//   D1 = sum_i inv_i delta_i,  Q = sum_i C_i,  R = sum_i (mean_i C_i - inv_i A_i / N):
+// the first term is what step_bwd_cross computes from the tensor this kernel leaves (D1 instead
+// of D), Q and R are two numbers per (element, block) left in `qr_out` for it.  The weights of
+// the taps that read the halo get x_h D1[c] - D2[c], D2 = sum_i mean_i inv_i delta_i (the halo
+// pass adds the first term, the second is subtracted once at the end).
+template <int BS, int CPT, int NSLOT, int ACT, bool LN, bool RES = false, bool NORM = false>
 __global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) __attribute__((amdgpu_waves_per_eu(2)))
 void step_bwd_fast(
     const float *__restrict__ weight, const float *__restrict__ bias,
     const float *__restrict__ scale, const float *__restrict__ x, const float *__restrict__ dy,
     float *__restrict__ dweight, float *__restrict__ dbias, float *__restrict__ dscale,
     float *__restrict__ dx, float *__restrict__ dsum_out, int B, int M, int N, int K, int inner,
-    int nblk, int nchunk, int chunk_len, int param_mode, int dx_accumulate, LnFold ln) {
+    int nblk, int nchunk, int chunk_len, int param_mode, int dx_accumulate, LnFold ln,
+    float norm_eps, float *__restrict__ qr_out) {
     using TL = Tile<BS, CPT>;
+    static_assert(!(NORM && (LN || RES)), "the folded LayerNorm comes without normalisation");
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int slot_floats = bwd_slot_floats<BS, CPT>(inner);
     // LN (the LayerNorm of the network body folded in, see LnFold): `dy` is the gradient with
@@ -935,6 +981,12 @@ void step_bwd_fast(
     const float *xhalo = win + (inner & 1) * TL::WIN;
     float *affine = lds + NSLOT * slot_floats;  // LN: gamma and beta of the window, packed
     const long cells = (long)M * N * K;
+    // NORM: the slot's statistics per iteration and the sums its waves exchange
+    constexpr int NW = bwd_norm_waves<BS, CPT>();
+    float *nstat = lds + NSLOT * slot_floats + pl.slot * bwd_norm_floats<BS, CPT>(inner);
+    float *ncommit = nstat + 4 * inner, *nown = ncommit + 4 * NW, *nrev = nown + 4 * NW;
+    const int wave_in_slot = TL::TPS >= 64 ? pl.lane / 64 : 0;
+    constexpr float inv_count = 1.f / TL::NWIN;
 
     // nw[t][c] belongs to the weight of the neighbour at c + off_t where that lies in this block,
     // and to this cell's own weight of tap t where it does not (see below)
@@ -995,6 +1047,19 @@ void step_bwd_fast(
                 v[t][c] = in_block(t, c) ? wl[(26 - t) * NC + lin + c + ((t / 9 - 1) * BS + ((t / 3) % 3 - 1)) * BS + (t % 3 - 1)]
                                          : 0.f;
         lds_barrier();  // the windows reuse this memory
+    }
+    // NORM: sum of a cell's 27 weights, and of those whose taps read the halo
+    float wsum[CPT], wout[CPT], zero[CPT], d2acc[CPT];
+    if (NORM) {
+#pragma unroll
+        for (int c = 0; c < CPT; ++c) {
+            wsum[c] = wout[c] = zero[c] = d2acc[c] = 0.f;
+#pragma unroll
+            for (int t = 0; t < 27; ++t) {
+                wsum[c] += w[t][c];
+                wout[c] += in_block(t, c) ? 0.f : w[t][c];
+            }
+        }
     }
     typename Fetch<TL>::Buf pre;
     if (ln_in && pl.slot == 0) {  // gamma and beta of the window, once per workgroup
@@ -1067,7 +1132,15 @@ void step_bwd_fast(
             if (RES) gin[c] = g[c];
         }
         if (ln_in) fx.commit_ln(win, pre, affine, nx_mean, nx_rstd);
-        else fx.commit(win, pre);
+        else if (NORM) {
+            float part[4];
+            fx.commit_sums(win, pre, part);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) part[q] = slot_wave_sum<TL::TPS>(part[q]);
+            if ((pl.lane & 63 & (TL::TPS - 1)) == 0)
+                *reinterpret_cast<float4 *>(ncommit + wave_in_slot * 4) =
+                    make_float4(part[0], part[1], part[2], part[3]);
+        } else fx.commit(win, pre);
     };
     if (ln_in) lds_barrier();  // gamma and beta windows
     if (s0 + pl.slot < s1) {
@@ -1080,12 +1153,14 @@ void step_bwd_fast(
     // the gradient of its own cells a thread leaves D = sum_i delta_i of them: what the cells
     // of neighbouring blocks and the weights of taps that read the frozen halo receive depends
     // on the iterations only through D, and a second kernel (step_bwd_cross) works it out.
-    float g_done[CPT], d_done[CPT];
+    float g_done[CPT], d_done[CPT], q_done = 0.f, r_done = 0.f;
     int done_s = -1;
     auto finish_done = [&]() {
         if (done_s < 0) return;
         const long o = (long)done_s * cells + pl.gc;
         store_cells<CPT>(dsum_out + o, d_done);
+        if (NORM && pl.lane == 0)
+            *reinterpret_cast<float2 *>(qr_out + ((long)done_s * nblk + blk) * 2) = make_float2(q_done, r_done);
         if (dx_accumulate) add_cells<CPT>(dx + o, g_done);
         else store_cells<CPT>(dx + o, g_done);
         if (RES && ln.g_out) store_cells<CPT>(ln.g_out + o, gin_done);
@@ -1099,24 +1174,65 @@ void step_bwd_fast(
         finish_done();
         if (s + NSLOT < s1) fetch_element(s + NSLOT);
         float cur[CPT];
+        float halo1 = 0.f, halo2 = 0.f, own1 = 0.f, own2 = 0.f;  // NORM: sums over the window
+        // NORM: statistics of the iteration at hand.  Every thread of the slot derives the same
+        // numbers from the same sums; one of them files them in LDS for the reverse sweep, which
+        // starts with those of the last iteration still in these registers (no barrier lies
+        // between that iteration and the sweep).
+        float mean = 0.f, sd = 1.f, inv = 1.f;
         if (active) {
 #pragma unroll
             for (int c = 0; c < CPT; ++c) cur[c] = win[pl.own + c];
+            if (NORM) {
+#pragma unroll
+                for (int q = 0; q < NW; ++q) {  // fixed order: every thread forms the same sums
+                    const float4 p4 = *reinterpret_cast<const float4 *>(ncommit + q * 4);
+                    halo1 += p4.x; halo2 += p4.y; own1 += p4.z; own2 += p4.w;
+                }
+            }
         }
 
         // ---- forward recompute, remembering x_i and u_i of the owned cells ----
         for (int it = 0; it < inner; ++it) {
             if (active) {
                 float u[CPT];
-                stencil<TL, CPT, kBwdDepth>(win + (it & 1) * TL::WIN, pl.row00, w, bv, u);
+                if (NORM) {
+                    if (it > 0) {
+                        own1 = own2 = 0.f;
+#pragma unroll
+                        for (int q = 0; q < NW; ++q) {
+                            const float2 p2 = *reinterpret_cast<const float2 *>(nown + ((it & 1) * NW + q) * 2);
+                            own1 += p2.x; own2 += p2.y;
+                        }
+                    }
+                    mean = (halo1 + own1) * inv_count;
+                    sd = sqrtf(fmaxf(fmaf(-mean, mean, (halo2 + own2) * inv_count), 0.f));
+                    inv = 1.f / (sd + norm_eps);
+                    if (pl.lane == 0) *reinterpret_cast<float4 *>(nstat + 4 * it) = make_float4(mean, sd, inv, 0.f);
+                    stencil<TL, CPT, kBwdDepth>(win + (it & 1) * TL::WIN, pl.row00, w, zero, u);
+#pragma unroll
+                    for (int c = 0; c < CPT; ++c) u[c] = fmaf(inv, fmaf(-mean, wsum[c], u[c]), bv[c]);
+                } else {
+                    stencil<TL, CPT, kBwdDepth>(win + (it & 1) * TL::WIN, pl.row00, w, bv, u);
+                }
                 float *h = hist + it * (TL::TPS * 2 * CPT);
                 store_cells<CPT>(h, cur);
                 store_cells<CPT>(h + TL::TPS * CPT, u);
                 if (it + 1 < inner) {
+                    float s1 = 0.f, s2 = 0.f;
 #pragma unroll
                     for (int c = 0; c < CPT; ++c) {
                         cur[c] = fmaf(rv[c], Act<ACT, float>::f(u[c]), cur[c]);
                         win[((it + 1) & 1) * TL::WIN + pl.own + c] = cur[c];
+                        s1 += cur[c];
+                        s2 = fmaf(cur[c], cur[c], s2);
+                    }
+                    if (NORM) {  // the owned cells' part of the next iteration's statistics
+                        s1 = slot_wave_sum<TL::TPS>(s1);
+                        s2 = slot_wave_sum<TL::TPS>(s2);
+                        if ((pl.lane & 63 & (TL::TPS - 1)) == 0)
+                            *reinterpret_cast<float2 *>(nown + (((it + 1) & 1) * NW + wave_in_slot) * 2) =
+                                make_float2(s1, s2);
                     }
                 } else {  // x_inner itself is never needed: that copy becomes the halo window
 #pragma unroll
@@ -1127,15 +1243,21 @@ void step_bwd_fast(
         }
 
         // ---- reverse sweep: delta window copy (it & 1) holds delta_it ----
-        float dsum[CPT], xi[CPT];
+        // NORM: dsum is D1, d2 is D2; x_i of the owned cells as the stencil saw it (xn); delta of
+        // the iteration; the halo brackets (wout is fixed, sout belongs to the element); Q and R
+        float dsum[CPT], xi[CPT], xn[CPT], d2[CPT], dlt[CPT], sout[CPT], q_sum = 0.f, r_sum = 0.f;
 #pragma unroll
-        for (int c = 0; c < CPT; ++c) dsum[c] = 0.f;
+        for (int c = 0; c < CPT; ++c) dsum[c] = d2[c] = sout[c] = 0.f;
         for (int it = inner - 1; it >= 0; --it) {
             if (active) {
                 const float *h = hist + it * (TL::TPS * 2 * CPT);
                 float u[CPT];
                 load_cells<CPT>(h, xi);
                 load_cells<CPT>(h + TL::TPS * CPT, u);
+                if (NORM && it < inner - 1) {
+                    const float4 st4 = *reinterpret_cast<const float4 *>(nstat + 4 * it);
+                    mean = st4.x; sd = st4.y; inv = st4.z;
+                }
 #pragma unroll
                 for (int c = 0; c < CPT; ++c) {
                     float f, d;
@@ -1143,7 +1265,15 @@ void step_bwd_fast(
                     const float delta = d * g[c] * rv[c];
                     dr[c] = fmaf(f, g[c], dr[c]);
                     db[c] += delta;
-                    dsum[c] += delta;
+                    if (NORM) {
+                        dlt[c] = delta;
+                        dsum[c] = fmaf(inv, delta, dsum[c]);
+                        d2[c] = fmaf(mean * inv, delta, d2[c]);
+                        xn[c] = (xi[c] - mean) * inv;
+                    } else {
+                        dsum[c] += delta;
+                        xn[c] = xi[c];
+                    }
                     dwin[(it & 1) * TL::WIN + pl.own + c] = delta;
                 }
             }
@@ -1163,6 +1293,14 @@ void step_bwd_fast(
                     });
             }
             lds_barrier();
+            if (NORM && active && it == inner - 1) {
+                // once per element: what the owned cells' taps into the halo see there (the
+                // halo window holds zeros in the block's cells, so the other taps add nothing)
+                stencil<TL, CPT, kBwdDepth>(xhalo, pl.row00, w, zero, sout);
+            }
+            float dn[CPT];  // NORM: gradient with respect to the normalised value of the owned cells
+#pragma unroll
+            for (int c = 0; c < CPT; ++c) dn[c] = 0.f;
             if (active) {
                 const float *dwn = dwin + (it & 1) * TL::WIN + pl.row00;
                 for_each_row<TL, CPT, kBwdDepth>(dwn, [&](int r, const float (&dv)[CPT + 2]) {
@@ -1170,10 +1308,47 @@ void step_bwd_fast(
                     for (int cc = 0; cc < 3; ++cc)
 #pragma unroll
                         for (int c = 0; c < CPT; ++c) {
-                            nw[r * 3 + cc][c] = fmaf(xi[c], dv[c + cc], nw[r * 3 + cc][c]);
-                            g[c] = fmaf(v[r * 3 + cc][c], dv[c + cc], g[c]);
+                            nw[r * 3 + cc][c] = fmaf(xn[c], dv[c + cc], nw[r * 3 + cc][c]);
+                            if (NORM) dn[c] = fmaf(v[r * 3 + cc][c], dv[c + cc], dn[c]);
+                            else g[c] = fmaf(v[r * 3 + cc][c], dv[c + cc], g[c]);
                         }
                 });
+            }
+            if (NORM) {
+                // A = sum dn and sum dn * x over the whole window, the halo through its brackets
+                float pa = 0.f, pb = 0.f;
+                if (active) {
+#pragma unroll
+                    for (int c = 0; c < CPT; ++c) {
+                        pa += fmaf(dlt[c], wout[c], dn[c]);
+                        pb += fmaf(dlt[c], sout[c], dn[c] * xi[c]);
+                    }
+                    pa = slot_wave_sum<TL::TPS>(pa);
+                    pb = slot_wave_sum<TL::TPS>(pb);
+                }
+                if (NW > 1) {
+                    if (active && (pl.lane & 63) == 0)
+                        *reinterpret_cast<float2 *>(nrev + wave_in_slot * 2) = make_float2(pa, pb);
+                    lds_barrier();
+                    if (active) {
+                        pa = pb = 0.f;
+#pragma unroll
+                        for (int q = 0; q < NW; ++q) {
+                            const float2 p2 = *reinterpret_cast<const float2 *>(nrev + q * 2);
+                            pa += p2.x; pb += p2.y;
+                        }
+                    }
+                }
+                if (active) {
+                    const float a_mean = pa * inv_count;
+                    const float proj = fmaf(-mean, pa, pb);  // sum dn (x - mean)
+                    const float coef = proj * inv * inv * inv_count / fmaxf(sd, 1e-30f);
+#pragma unroll
+                    for (int c = 0; c < CPT; ++c)
+                        g[c] += fmaf(inv, dn[c] - a_mean, -(xi[c] - mean) * coef);
+                    q_sum += coef;
+                    r_sum += fmaf(mean, coef, -inv * a_mean);
+                }
             }
         }
 
@@ -1184,6 +1359,11 @@ void step_bwd_fast(
             g_done[c] = g[c];
             d_done[c] = dsum[c];
             if (RES) gin_done[c] = gin[c];
+            if (NORM && active) d2acc[c] += d2[c];
+        }
+        if (NORM) {
+            q_done = q_sum;
+            r_done = r_sum;
         }
         // the x windows are free (the reverse sweep does not read them): commit the next one
         if (s + NSLOT < s1) take_element();
@@ -1214,8 +1394,15 @@ void step_bwd_fast(
                 reduce(dgam[c]);
                 reduce(dbet[c]);
             }
+            if (NORM) reduce(d2acc[c]);
         }
         if (pl.slot != 0) return;
+    }
+    if (NORM) {  // the taps that read the halo: x_h D1 was added per element, D2 is still owed
+#pragma unroll
+        for (int t = 0; t < 27; ++t)
+#pragma unroll
+            for (int c = 0; c < CPT; ++c) nw[t][c] -= in_block(t, c) ? 0.f : d2acc[c];
     }
     commit_grads<27, CPT>(dweight, nw, param_mode, owner_of, always);
     float one[1][CPT];
@@ -1262,18 +1449,25 @@ void step_bwd_fast(
 // RES (with LN): the outer_residual form of the loop, see LnFold: what is completed here is
 // the gradient with respect to n = LayerNorm(x), and what goes to dx (and into the sums) is
 // dn = that minus G', the gradient with respect to the step's output.
-template <int BS, int NSLOT, int E, bool LN, bool RES = false>
+// NORM (per-window normalisation, see step_bwd_fast): `dsum` holds D1, and a cell that lies in
+// the halo of a neighbouring block a additionally receives R_a - x Q_a from it, Q and R being
+// the two numbers per (element, block) that step_bwd_fast left in `qr`.  The row threads add
+// that: they load their row of x, and the (Q, R) of the 26 neighbours of the block travel
+// through LDS with the D windows.
+template <int BS, int NSLOT, int E, bool LN, bool RES = false, bool NORM = false>
 __global__ __launch_bounds__((6 * BS * BS * NSLOT)) __attribute__((amdgpu_waves_per_eu(3)))
 void step_bwd_cross(
     const float *__restrict__ weight, const float *__restrict__ x, const float *__restrict__ dsum,
     float *__restrict__ dx, int B, int M, int N, int K, int nblk, int nchunk, int chunk_len,
-    LnFold ln) {
+    LnFold ln, const float *__restrict__ qr) {
     using TL = Tile<BS, 1>;  // window geometry only
     constexpr int FS = BS * BS, TPS = 6 * FS;
     constexpr int PAIR = TL::WIN;                  // the D window of one element
     constexpr int STAGE = E * PAIR;                // the E elements of a round
-    constexpr int SLOT = 2 * STAGE + 2 * E * TPS;  // two stages, two slabs
+    constexpr int QRS = NORM ? 2 * E * 27 * 2 : 0; // NORM: (Q, R) of the neighbours, two stages
+    constexpr int SLOT = 2 * STAGE + 2 * E * TPS + QRS;  // two stages, two slabs
     __shared__ __attribute__((aligned(16))) float lds[NSLOT * SLOT];
+    static_assert(!(NORM && (LN || RES)), "the folded LayerNorm comes without normalisation");
 
     int blk, chunk;
     if (!split_block_id(blockIdx.x, nblk, nchunk, blk, chunk)) return;  // grid padding
@@ -1302,6 +1496,16 @@ void step_bwd_cross(
     const bool ri_edge = ri == 0 || ri == BS - 1, rj_edge = rj == 0 || rj == BS - 1;
 
     const bool ln_in = LN && ln.x_stats != nullptr;
+    // NORM: thread n < 27 fetches (Q, R) of the neighbouring block at offset
+    // (n/9 - 1, (n/3)%3 - 1, n%3 - 1); blocks outside the grid (and the block itself) count as 0
+    float *qrs = slabs + 2 * E * TPS;  // [2 stages][E][27][2]
+    int qr_blk = -1;
+    if (NORM && lane < 27 && lane != 13) {
+        const int mb = M / BS;
+        const int bi = blk / (kb * nb) + lane / 9 - 1, bj = (blk / kb) % nb + (lane / 3) % 3 - 1,
+                  bk = blk % kb + lane % 3 - 1;
+        if (bi >= 0 && bi < mb && bj >= 0 && bj < nb && bk >= 0 && bk < kb) qr_blk = (bi * nb + bj) * kb + bk;
+    }
     float vx[9];
     float grw[BS];  // LN, row threads: gamma of their row
     if (ln_in && is_row) load_cells<BS>(ln.gamma + grow, grw);
@@ -1331,6 +1535,7 @@ void step_bwd_cross(
     // element e of round r of this slot; past the end of the chunk it is not `real`
     auto sample = [&](int r, int e) { return s0 + (r * E + e) * NSLOT + slot; };
     Buf pd[E];
+    float2 pq[E];  // NORM: (Q, R) of this thread's neighbour block
     // Loads and commits are unconditional (past the end of the chunk they repeat its last
     // element, which nobody then uses): with branches around them the compiler cannot count the
     // loads in flight and waits for ALL of them wherever it needs one.
@@ -1340,12 +1545,19 @@ void step_bwd_cross(
             const int sc = min(sample(r, e), s1 - 1);
             const long at = (long)sc * cells;
             fx.fetch(dsum + at, pd[e]);
+            if (NORM) {  // every thread loads (a valid address always), the commit selects
+                const float *from = qr + ((long)sc * nblk + (qr_blk >= 0 ? qr_blk : blk)) * 2;
+                pq[e] = make_float2(from[0], from[1]);
+            }
         }
     };
     auto commit_round = [&](int st) {
 #pragma unroll
         for (int e = 0; e < E; ++e) {
             fx.template commit<1>(stages + st * STAGE + e * PAIR, pd[e]);
+            if (NORM && lane < 27)
+                *reinterpret_cast<float2 *>(qrs + ((st * E + e) * 27 + lane) * 2) =
+                    qr_blk >= 0 ? pq[e] : make_float2(0.f, 0.f);
         }
     };
     float gx[E][BS];  // row threads: dx of their row so far (the own block's part)
@@ -1377,6 +1589,33 @@ void step_bwd_cross(
                 if (RES) {
 #pragma unroll
                     for (int c = 0; c < BS; ++c) gx[e][c] -= gr[e][c];
+                }
+                if (NORM) {
+                    // neighbours that have this row in their halo, by their offset along K:
+                    // (0, 0), (ei, 0), (0, ej), (ei, ej) with ei, ej the side of the block the
+                    // row lies on, if any; along K only the row's end cells are concerned
+                    const float *q27 = qrs + (st * E + e) * 27 * 2;
+                    const int ei = ri == 0 ? -1 : ri == BS - 1 ? 1 : 0, ej = rj == 0 ? -1 : rj == BS - 1 ? 1 : 0;
+                    float rq[3], rr[3];
+#pragma unroll
+                    for (int dk = 0; dk < 3; ++dk) {
+                        float sq = 0.f, sr = 0.f;
+                        auto add = [&](int a, int b) {
+                            const float2 v2 = *reinterpret_cast<const float2 *>(q27 + (((a + 1) * 3 + (b + 1)) * 3 + dk) * 2);
+                            sq += v2.x;
+                            sr += v2.y;
+                        };
+                        if (dk != 1) add(0, 0);
+                        if (ei != 0) add(ei, 0);
+                        if (ej != 0) add(0, ej);
+                        if (ei != 0 && ej != 0) add(ei, ej);
+                        rq[dk] = sq;
+                        rr[dk] = sr;
+                    }
+#pragma unroll
+                    for (int c = 0; c < BS; ++c) gx[e][c] += fmaf(-xr[e][c], rq[1], rr[1]);
+                    gx[e][0] += fmaf(-xr[e][0], rq[0], rr[0]);
+                    gx[e][BS - 1] += fmaf(-xr[e][BS - 1], rq[2], rr[2]);
                 }
                 if (s < s1) store_cells<BS>(dx + (long)s * cells + grow, gx[e]);
                 if (ln_in) {
@@ -1412,6 +1651,7 @@ void step_bwd_cross(
                 const int sc = min(sample(r, e), s1 - 1);
                 load_cells<BS>(dx + (long)sc * cells + grow, gx[e]);
                 if (RES) load_cells<BS>(ln.g_rows + (long)sc * cells + grow, gr[e]);
+                if (NORM) load_cells<BS>(x + (long)sc * cells + grow, xr[e]);
                 if (ln_in) {
                     load_cells<BS>(x + (long)sc * cells + grow, xr[e]);
                     xmean[e] = load_ahead(ln.x_stats, 2 * sc);
@@ -1537,12 +1777,12 @@ constexpr size_t kMaxLds = 160 * 1024;
 constexpr int kCrossSlots8 = 1, kCrossElems8 = 2;  // bs=8: 384 threads, one wave per face
 constexpr int kCrossSlots4 = 2, kCrossElems4 = 2;  // bs=4: two slots of 96 threads
 
-template <int BS, int CPT, int NSLOT, int ACT, bool LN, bool RES = false>
+template <int BS, int CPT, int NSLOT, int ACT, bool LN, bool RES = false, bool NORM = false>
 int launch_bwd_ln(const StepArgs &a, hipStream_t st) {
     using TL = Tile<BS, CPT>;
     const long cells = (long)a.M * a.N * a.K;
-    const size_t lds = bwd_lds_bytes<BS, CPT, NSLOT>(a.inner, LN);
-    auto kern = step_bwd_fast<BS, CPT, NSLOT, ACT, LN, RES>;
+    const size_t lds = bwd_lds_bytes<BS, CPT, NSLOT>(a.inner, LN, NORM);
+    auto kern = step_bwd_fast<BS, CPT, NSLOT, ACT, LN, RES, NORM>;
     static bool big_lds_enabled = false;            // per instantiation
     static int per_cu_cache[kMaxBackwardIters + 1];  // per instantiation, by inner iterations
     if (lds > 64 * 1024 && !big_lds_enabled) {
@@ -1580,23 +1820,27 @@ int launch_bwd_ln(const StepArgs &a, hipStream_t st) {
         }
     }
     const int dx_accumulate = (a.flags & GRIDNET_OVERWRITE_DX) ? 0 : 1;
+    // NORM: (Q, R) per (element, block), behind the D tensor in the workspace
+    float *qr = NORM ? (float *)a.workspace + (size_t)a.B * cells : nullptr;
     hipLaunchKernelGGL(kern, dim3(padded_grid(p.nblk, p.nchunk)), dim3(TL::TPS * NSLOT), lds, st,
                        (const float *)a.weight, (const float *)a.bias, (const float *)a.scale,
                        (const float *)a.x, (const float *)a.dy, (float *)a.dweight, (float *)a.dbias,
                        (float *)a.dscale, (float *)a.dx, (float *)a.workspace, a.B, a.M, a.N, a.K,
-                       a.inner, p.nblk, p.nchunk, p.chunk_len, param_mode, dx_accumulate, a.ln);
+                       a.inner, p.nblk, p.nchunk, p.chunk_len, param_mode, dx_accumulate, a.ln,
+                       (float)a.eps, qr);
     if (int rc = check_launch("step_bwd_fast")) return rc;
     // same blocks, same batch chunks; the parameter gradients are complete, dx is not yet
     constexpr int XSLOT = BS == 8 ? kCrossSlots8 : kCrossSlots4;
     constexpr int XE = BS == 8 ? kCrossElems8 : kCrossElems4;
-    hipLaunchKernelGGL((step_bwd_cross<BS, XSLOT, XE, LN, RES>), dim3(padded_grid(p.nblk, p.nchunk)),
+    hipLaunchKernelGGL((step_bwd_cross<BS, XSLOT, XE, LN, RES, NORM>), dim3(padded_grid(p.nblk, p.nchunk)),
                        dim3(6 * BS * BS * XSLOT), 0, st, (const float *)a.weight,
                        (const float *)a.x, (const float *)a.workspace, (float *)a.dx, a.B, a.M, a.N,
-                       a.K, p.nblk, p.nchunk, p.chunk_len, a.ln);
+                       a.K, p.nblk, p.nchunk, p.chunk_len, a.ln, (const float *)qr);
     if (int rc = check_launch("step_bwd_cross")) return rc;
     return GRIDNET_OK;
 }
 template <int BS, int CPT, int NSLOT, int ACT> int launch_bwd(const StepArgs &a, hipStream_t st) {
+    if (a.normalize) return launch_bwd_ln<BS, CPT, NSLOT, ACT, false, false, true>(a, st);
     if (a.ln.gamma && a.ln.residual) return launch_bwd_ln<BS, CPT, NSLOT, ACT, true, true>(a, st);
     if (a.ln.gamma) return launch_bwd_ln<BS, CPT, NSLOT, ACT, true>(a, st);
     return launch_bwd_ln<BS, CPT, NSLOT, ACT, false>(a, st);
@@ -1637,20 +1881,23 @@ int step_fast_backward_parts(int block_size) { return block_size * block_size / 
 
 bool step_fast_supports(const StepArgs &a, bool backward) {
     if (a.dtype != GRIDNET_F32) return false;
-    if (a.normalize && (backward || a.ln.gamma)) return false;  // forward only, plain step only
+    if (a.normalize && a.ln.gamma) return false;  // the folded LayerNorm: plain step only
     if (a.block_size != 4 && a.block_size != 8) return false;
     if (backward) {
         const bool ln = a.ln.gamma != nullptr;
-        const size_t lds = a.block_size == 8 ? bwd_lds_bytes<8, kBwdCpt8, kBwdSlots8>(a.inner, ln)
-                                             : bwd_lds_bytes<4, kBwdCpt4, kBwdSlots4>(a.inner, ln);
+        const size_t lds = a.block_size == 8
+                               ? bwd_lds_bytes<8, kBwdCpt8, kBwdSlots8>(a.inner, ln, a.normalize)
+                               : bwd_lds_bytes<4, kBwdCpt4, kBwdSlots4>(a.inner, ln, a.normalize);
         if (lds > kMaxLds) return false;
     }
     return true;
 }
 
 size_t step_fast_backward_workspace(const StepArgs &a) {
-    // D = sum_i delta_i of every cell, handed from step_bwd_fast to step_bwd_cross
-    return (size_t)a.B * a.M * a.N * a.K * sizeof(float);
+    // D = sum_i delta_i of every cell, handed from step_bwd_fast to step_bwd_cross; with
+    // normalize, two more numbers per (element, block)
+    const size_t nblk = (size_t)(a.M / a.block_size) * (a.N / a.block_size) * (a.K / a.block_size);
+    return ((size_t)a.B * a.M * a.N * a.K + (a.normalize ? (size_t)a.B * nblk * 2 : 0)) * sizeof(float);
 }
 
 int step_forward_fast(const StepArgs &a, hipStream_t st) { return dispatch<false>(a, st); }

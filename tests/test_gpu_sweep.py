@@ -62,6 +62,46 @@ def test_random_step_tuned_fp32_against_generic_fp64(seed):
                      what=name)
 
 
+def draw_normalized(seed):
+    if seed == 0:  # the draw that once showed a missing barrier in the tuned backward
+        return (24, 24, 24), 8, 40, 1, "tanh"
+    rng = random.Random(7000 + seed)
+    bs = rng.choice((4, 8))
+    shape = tuple(bs * rng.randint(1, 3) for _ in range(3))
+    return shape, bs, rng.choice((1, 2, 5, 17, 40)), rng.choice((0, 1, 2, 3, 5)), rng.choice(SMOOTH)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_normalized_step_tuned_fp32_against_generic_fp64(seed):
+    """normalize=True: the tuned kernels keep running sums for the window statistics and hand
+    two numbers per (element, block) to the cross-block kernel; the generic kernels (the only
+    implementation in fp64) reduce over the window twice per iteration."""
+    import gridnet_cuda
+
+    shape, bs, batch, inner, activation = draw_normalized(seed)
+    print(f"sweep normalized seed={seed} shape={shape} bs={bs} B={batch} inner={inner} "
+          f"act={activation}", flush=True)
+    w, b, r = make_params(shape, seed=7100 + seed)
+    x, gy = make_acts(batch, shape, seed=7200 + seed), make_acts(batch, shape, seed=7300 + seed)
+
+    def call(dtype):
+        tw, tb, tr, tx, tgy = (t.to(device=DEV, dtype=dtype) for t in (w, b, r, x, gy))
+        y = torch.full_like(tx, float("nan"))
+        gridnet_cuda.forward(tw, tb, tr, tx, y, inner, bs, 1e-5, True, activation)
+        outs = [torch.zeros_like(t) for t in (tw, tb, tr, tx)]
+        gridnet_cuda.backward(tw, tb, tr, tx, tgy, *outs, inner, bs, 1e-5, True, activation)
+        return [y] + outs
+
+    fast, slow = call(torch.float32), call(torch.float64)
+    # the division by (std + eps) and the two window sums of the backward double the rounding
+    # of a plain step: twice the bar's tolerances here, the bar itself against the oracle on
+    # the reference's own matrix (test_gpu_step.py)
+    summed = 2e-5 * max(1.0, math.sqrt(batch * max(inner, 1) / 2))
+    for name, got, want in zip(("y", "dweight", "dbias", "dscale", "dx"), fast, slow):
+        assert torch.isfinite(got).all(), name
+        assert_close(got, want, rtol=2e-4, atol=summed if name != "y" else 2e-5, what=name)
+
+
 def draw_chain(seed):
     rng = random.Random(100 + seed)
     bs = rng.choice((4, 8))
