@@ -23,11 +23,11 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def run(dtype, w, b, r, x, gy, inner, bs, activation):
+def run(dtype, w, b, r, x, gy, inner, bs, activation, normalize=False):
     from gridnet_amd.backend_cuda import GridnetCudaOp
 
     leaves = [t.to(device=DEV, dtype=dtype).requires_grad_(True) for t in (w, b, r, x)]
-    y = GridnetCudaOp.apply(*leaves, inner, bs, 1e-5, False, activation)
+    y = GridnetCudaOp.apply(*leaves, inner, bs, 1e-5, normalize, activation)
     grads = torch.autograd.grad(y, leaves, gy.to(device=DEV, dtype=dtype))
     return (y.detach(), *grads)
 
@@ -70,3 +70,23 @@ def test_tuned_fp32_against_generic_fp64(shape, bs, inner, batch, activation, sc
     for name, got, want in zip(("y", "dweight", "dbias", "dscale", "dx"), fast, slow):
         assert_close(got, want, atol=summed if name in ("dweight", "dbias", "dscale") else 1e-5,
                      what=name)
+
+
+@pytest.mark.parametrize("shape,bs,inner,batch", [
+    ((64, 64, 64), 8, 4, 32),   # the graded shape with the reference's default normalize=True
+    ((64, 64, 64), 4, 3, 5),    # 4096 blocks of 4^3
+    ((24, 40, 16), 8, 2, 70),   # fewer blocks than CUs: batch split over workgroups
+])
+def test_tuned_fp32_against_generic_fp64_normalized(shape, bs, inner, batch):
+    """normalize=True at full size (silu, the reference's default activation).  Twice the bar's
+    tolerances, as in the sweep of small shapes: the division by (std + eps) and the two window
+    sums of the backward double the rounding of a plain step."""
+    print(f"cross-check normalized shape={shape} bs={bs} inner={inner} B={batch}", flush=True)
+    w, b, r = make_params(shape, seed=41)
+    x, gy = make_acts(batch, shape, seed=42), make_acts(batch, shape, seed=43)
+    fast = run(torch.float32, w, b, r, x, gy, inner, bs, "silu", True)
+    slow = run(torch.float64, w, b, r, x, gy, inner, bs, "silu", True)
+    summed = 2e-5 * max(1.0, math.sqrt(batch * inner / 2))
+    for name, got, want in zip(("y", "dweight", "dbias", "dscale", "dx"), fast, slow):
+        assert torch.isfinite(got).all(), name
+        assert_close(got, want, rtol=2e-4, atol=2e-5 if name in ("y", "dx") else summed, what=name)
