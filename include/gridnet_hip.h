@@ -91,7 +91,7 @@ size_t gridnet_hip_backward_workspace_bytes(int dtype, int B, int M, int N, int 
  * (bound as `backward`, src/gridnet_cuda.cpp:91-131,191).  Recomputes the inner forward
  * from x; inner <= 32.  dweight [27,M,N,K], dbias, dscale [M,N,K] are summed over the batch;
  * dx [B,M,N,K].  `workspace` must hold gridnet_hip_backward_workspace_bytes() bytes (contents
- * need no initialisation; 256-byte aligned).
+ * need no initialisation).
  */
 int gridnet_hip_backward(int dtype, const void *weight, const void *bias, const void *scale,
                          const void *x, const void *dy, void *dweight, void *dbias,
