@@ -64,7 +64,7 @@ using namespace gridnet;
 
 extern "C" {
 
-int gridnet_hip_version(void) { return 3; }  // 2: fused body entry points; 3: residual forward and backward
+int gridnet_hip_version(void) { return 4; }  // 2: fused body; 3: residual forward and backward; 4: gated backward takes a workspace
 
 const char *gridnet_hip_last_error(void) { return error_buffer(); }
 
@@ -135,23 +135,44 @@ int gridnet_hip_forward_gated(int dtype, const void *weight, const void *bias, c
     a.B = B; a.M = M; a.N = N; a.K = K; a.inner = inner; a.block_size = block_size;
     a.activation = activation;
     if (int rc = check_step(a, false, true)) return rc;
+    if ((long)M * N * K * 54 >= (1L << 31))
+        return fail(GRIDNET_ERR_ARGUMENT, "grid too large: 54*M*N*K must be below 2^31");
     if (B == 0) return GRIDNET_OK;
+    if (gated_fast_supports(a, false)) return gated_forward_fast(a, (hipStream_t)stream);
     return gated_forward(a, (hipStream_t)stream);
+}
+
+size_t gridnet_hip_backward_gated_workspace_bytes(int dtype, int B, int M, int N, int K, int inner,
+                                                  int block_size) {
+    StepArgs a{};
+    a.dtype = dtype; a.B = B; a.M = M; a.N = N; a.K = K; a.inner = inner;
+    a.block_size = block_size; a.activation = GRIDNET_ACT_RELU;
+    if (B <= 0 || M <= 0 || N <= 0 || K <= 0) return 0;
+    if (gated_fast_supports(a, true)) return gated_fast_backward_workspace(a);
+    return 0;
 }
 
 int gridnet_hip_backward_gated(int dtype, const void *weight, const void *bias, const void *x,
                                const void *dy, void *dweight, void *dbias, void *dx, int B, int M,
                                int N, int K, int inner, int block_size, int activation, int flags,
-                               void *stream) {
+                               void *workspace, size_t workspace_bytes, void *stream) {
     StepArgs a{};
     a.dtype = dtype; a.weight = weight; a.bias = bias; a.x = x; a.dy = dy;
     a.dweight = dweight; a.dbias = dbias; a.dx = dx;
     a.B = B; a.M = M; a.N = N; a.K = K; a.inner = inner; a.block_size = block_size;
     a.activation = activation; a.flags = flags;
+    a.workspace = workspace; a.workspace_bytes = workspace_bytes;
     if (int rc = check_step(a, true, true)) return rc;
     if ((long)M * N * K * 54 >= (1L << 31))
         return fail(GRIDNET_ERR_ARGUMENT, "grid too large: 54*M*N*K must be below 2^31");
     if (B == 0) return GRIDNET_OK;
+    if (gated_fast_supports(a, true)) {
+        const size_t need = gated_fast_backward_workspace(a);
+        if (!workspace || workspace_bytes < need)
+            return fail(GRIDNET_ERR_WORKSPACE, "backward needs %zu bytes of workspace, got %zu", need,
+                        workspace ? workspace_bytes : (size_t)0);
+        return gated_backward_fast(a, (hipStream_t)stream);
+    }
     return gated_backward(a, (hipStream_t)stream);
 }
 

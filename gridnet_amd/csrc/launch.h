@@ -85,6 +85,15 @@ int step_fast_forward_parts(int block_size);   // (mean, M2) pairs, each over fo
 int step_fast_forward_part_count(int block_size);
 int step_fast_backward_parts(int block_size);  // (sum g, sum g*xhat) pairs
 
+// step_fast.hip: the cross-block kernel on two weight sets, for gated_fast.hip
+int gated_cross_launch(const StepArgs &a, const float *dsum, int nchunk, int chunk_len, hipStream_t st);
+
+// gated_fast.hip: fp32, block sizes 4 and 8, as many inner iterations as the LDS holds
+bool gated_fast_supports(const StepArgs &a, bool backward);
+size_t gated_fast_backward_workspace(const StepArgs &a);
+int gated_forward_fast(const StepArgs &a, hipStream_t st);
+int gated_backward_fast(const StepArgs &a, hipStream_t st);
+
 // gated_generic.hip (weight [27,2,M,N,K], bias [2,M,N,K]; scale, eps, normalize unused)
 int gated_forward(const StepArgs &a, hipStream_t st);
 int gated_backward(const StepArgs &a, hipStream_t st);

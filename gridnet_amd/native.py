@@ -28,6 +28,7 @@ EXPORTS = (
     "gridnet_hip_backward_workspace_bytes",
     "gridnet_hip_backward",
     "gridnet_hip_forward_gated",
+    "gridnet_hip_backward_gated_workspace_bytes",
     "gridnet_hip_backward_gated",
     "gridnet_hip_layernorm_workspace_bytes",
     "gridnet_hip_layernorm_forward",
@@ -68,8 +69,10 @@ def _load():
                                          p, z, p]
     lib.gridnet_hip_forward_gated.restype = i
     lib.gridnet_hip_forward_gated.argtypes = [i, p, p, p, p, i, i, i, i, i, i, i, p]
+    lib.gridnet_hip_backward_gated_workspace_bytes.restype = z
+    lib.gridnet_hip_backward_gated_workspace_bytes.argtypes = [i, i, i, i, i, i, i]
     lib.gridnet_hip_backward_gated.restype = i
-    lib.gridnet_hip_backward_gated.argtypes = [i, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, p]
+    lib.gridnet_hip_backward_gated.argtypes = [i, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, p, z, p]
     lib.gridnet_hip_layernorm_workspace_bytes.restype = z
     lib.gridnet_hip_layernorm_workspace_bytes.argtypes = [i, i, l]
     lib.gridnet_hip_layernorm_forward.restype = i

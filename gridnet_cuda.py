@@ -83,9 +83,13 @@ def backward_gated(weight, bias, initActivations, outGrads, weightGradOut, biasG
         _n.check_input(t, name)
     act = _n.activation_id(activation)
     B, M, N, K = initActivations.shape
+    dt = _n.dtype_id(weight)
     with torch.cuda.device(weight.device):
+        nbytes = _n.lib.gridnet_hip_backward_gated_workspace_bytes(
+            dt, B, M, N, K, int(innerIterations), int(blockSize))
+        ws = _n.workspace(nbytes, weight.device)
         _n.check(_n.lib.gridnet_hip_backward_gated(
-            _n.dtype_id(weight), weight.data_ptr(), bias.data_ptr(), initActivations.data_ptr(),
+            dt, weight.data_ptr(), bias.data_ptr(), initActivations.data_ptr(),
             outGrads.data_ptr(), weightGradOut.data_ptr(), biasGradOut.data_ptr(),
             activationsGradOut.data_ptr(), B, M, N, K, int(innerIterations), int(blockSize), act, 0,
-            _n.current_stream(weight)))
+            ws.data_ptr(), nbytes, _n.current_stream(weight)))

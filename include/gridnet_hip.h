@@ -105,16 +105,20 @@ int gridnet_hip_backward(int dtype, const void *weight, const void *bias, const 
  * gated_gridnet_cuda_forward / gated_gridnet_cuda_backward, src/gridnet_cuda_kernels.cu:853-930
  * (bound as `forward_gated` / `backward_gated`, src/gridnet_cuda.cpp:133-186,192-193).
  * Backward: inner <= 32; dweight [27,2,M,N,K], dbias [2,M,N,K] summed over the batch; flags as
- * for gridnet_hip_backward.  No workspace.
+ * for gridnet_hip_backward; `workspace` must hold gridnet_hip_backward_gated_workspace_bytes()
+ * bytes (may be 0; contents need no initialisation).
  */
 int gridnet_hip_forward_gated(int dtype, const void *weight, const void *bias, const void *x,
                               void *y, int B, int M, int N, int K, int inner, int block_size,
                               int activation, void *stream);
 
+size_t gridnet_hip_backward_gated_workspace_bytes(int dtype, int B, int M, int N, int K, int inner,
+                                                  int block_size);
+
 int gridnet_hip_backward_gated(int dtype, const void *weight, const void *bias, const void *x,
                                const void *dy, void *dweight, void *dbias, void *dx, int B, int M,
                                int N, int K, int inner, int block_size, int activation, int flags,
-                               void *stream);
+                               void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * Per-sample LayerNorm over all n = M*N*K cells with elementwise affine, the op the callers

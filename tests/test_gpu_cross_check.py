@@ -90,3 +90,30 @@ def test_tuned_fp32_against_generic_fp64_normalized(shape, bs, inner, batch):
     for name, got, want in zip(("y", "dweight", "dbias", "dscale", "dx"), fast, slow):
         assert torch.isfinite(got).all(), name
         assert_close(got, want, rtol=2e-4, atol=2e-5 if name in ("y", "dx") else summed, what=name)
+
+
+@pytest.mark.parametrize("shape,bs,inner,batch", [
+    ((64, 64, 64), 8, 4, 32),   # one workgroup of 512 threads per block owns the whole batch
+    ((64, 64, 64), 4, 3, 5),    # 4096 blocks, two 64-thread slots per workgroup
+    ((24, 40, 16), 8, 2, 70),   # fewer blocks than CUs: batch split, parameter gradients by atomics
+])
+def test_gated_tuned_fp32_against_generic_fp64(shape, bs, inner, batch):
+    """The gated variant at full size (tanh, the activation the reference's scripts pair it with)."""
+    from gridnet_amd.backend_cuda import GatedGridnetCudaOp
+
+    print(f"cross-check gated shape={shape} bs={bs} inner={inner} B={batch}", flush=True)
+    gen = torch.Generator().manual_seed(51)
+    w = torch.randn(27, 2, *shape, generator=gen) / 27 ** 0.5
+    b = 0.1 * torch.randn(2, *shape, generator=gen)
+    x, gy = make_acts(batch, shape, seed=52), make_acts(batch, shape, seed=53)
+
+    def call(dtype):
+        leaves = [t.to(device=DEV, dtype=dtype).requires_grad_(True) for t in (w, b, x)]
+        y = GatedGridnetCudaOp.apply(*leaves, inner, bs, "tanh")
+        return (y.detach(), *torch.autograd.grad(y, leaves, gy.to(device=DEV, dtype=dtype)))
+
+    fast, slow = call(torch.float32), call(torch.float64)
+    summed = 1e-5 * max(1.0, math.sqrt(batch * inner / 2))
+    for name, got, want in zip(("y", "dweight", "dbias", "dx"), fast, slow):
+        assert torch.isfinite(got).all(), name
+        assert_close(got, want, atol=summed if name in ("dweight", "dbias") else 1e-5, what=name)

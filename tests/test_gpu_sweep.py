@@ -6,7 +6,7 @@ stores for the parameter gradients), so a fixed list of cases exercises a fixed 
 Here grid, block size, batch, inner iterations, activation and the accumulate/overwrite flags are
 drawn at random (fixed seeds) and every draw is held to the generic kernels run in fp64 on the
 same fp32 inputs -- the two share no device code, and each is held to the CPU oracle elsewhere
-(test_gpu_step.py).  A second sweep holds the chain with the LayerNorm folded into the step
+(test_gpu_step.py); likewise with normalize=True and for the gated variant of the step.  A second sweep holds the chain with the LayerNorm folded into the step
 kernels to the op-by-op chain of the same library, in both shapes of the loop."""
 
 import math
@@ -100,6 +100,43 @@ def test_random_normalized_step_tuned_fp32_against_generic_fp64(seed):
     for name, got, want in zip(("y", "dweight", "dbias", "dscale", "dx"), fast, slow):
         assert torch.isfinite(got).all(), name
         assert_close(got, want, rtol=2e-4, atol=summed if name != "y" else 2e-5, what=name)
+
+
+def draw_gated(seed):
+    rng = random.Random(8000 + seed)
+    bs = rng.choice((4, 8))
+    shape = tuple(bs * rng.randint(1, 3) for _ in range(3))
+    return (shape, bs, rng.choice((1, 2, 5, 17, 40, 64)), rng.choice((0, 1, 2, 3, 5)),
+            rng.choice(SMOOTH), rng.random() < 0.5)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_gated_step_tuned_fp32_against_generic_fp64(seed):
+    import gridnet_cuda
+
+    shape, bs, batch, inner, activation, preset = draw_gated(seed)
+    print(f"sweep gated seed={seed} shape={shape} bs={bs} B={batch} inner={inner} act={activation} "
+          f"preset={preset}", flush=True)
+    gen = torch.Generator().manual_seed(8100 + seed)
+    w = torch.randn(27, 2, *shape, generator=gen) / 27 ** 0.5
+    b = 0.1 * torch.randn(2, *shape, generator=gen)
+    x, gy = make_acts(batch, shape, seed=8200 + seed), make_acts(batch, shape, seed=8300 + seed)
+    start = [make_acts(1, t.shape, seed=8400 + seed + i)[0] if preset else torch.zeros_like(t)
+             for i, t in enumerate((w, b, x))]
+
+    def call(dtype):
+        tw, tb, tx, tgy = (t.to(device=DEV, dtype=dtype) for t in (w, b, x, gy))
+        y = torch.full_like(tx, float("nan"))
+        gridnet_cuda.forward_gated(tw, tb, tx, y, inner, bs, activation)
+        outs = [t.to(device=DEV, dtype=dtype) for t in start]
+        gridnet_cuda.backward_gated(tw, tb, tx, tgy, *outs, inner, bs, activation)
+        return [y] + outs
+
+    fast, slow = call(torch.float32), call(torch.float64)
+    summed = 1e-5 * max(1.0, math.sqrt(batch * max(inner, 1) / 2))
+    for name, got, want in zip(("y", "dweight", "dbias", "dx"), fast, slow):
+        assert torch.isfinite(got).all(), name
+        assert_close(got, want, atol=summed if name in ("dweight", "dbias") else 1e-5, what=name)
 
 
 def draw_chain(seed):
