@@ -45,6 +45,27 @@ def test_gated_parity(dtype, rtol, atol, shape, bs, inner, activation):
         assert_close(g, e, rtol, atol, name)
 
 
+@pytest.mark.parametrize("inner", [16, 21, 22, 32])
+@pytest.mark.parametrize("bs", [8, 4])
+def test_gated_deep_inner_iterations(bs, inner):
+    """Up to the reference's limit of 32 (src/gridnet_cuda_kernels.cu:925).  With 8^3 blocks the
+    tuned backward keeps the history of 21 iterations in LDS; beyond that the generic kernels
+    take over, and the results must not show where."""
+    from gridnet_amd.backend_cuda import GatedGridnetCudaOp
+
+    print(f"gated deep bs={bs} inner={inner}", flush=True)
+    w, b, x, gy = make((8, 8, 16), torch.float32, seed=3, scale=0.1)
+    leaves = [t.to(DEV).requires_grad_(True) for t in (w, b, x)]
+    y = GatedGridnetCudaOp.apply(*leaves, inner, bs, "tanh")
+    grads = torch.autograd.grad(y, leaves, gy.to(DEV))
+    ref = [t.double().requires_grad_(True) for t in (w, b, x)]
+    ey = gated_step_fast(*ref, inner, bs, "tanh")
+    egrads = torch.autograd.grad(ey, ref, gy.double())
+    assert_close(y, ey, what="y")
+    for name, g, e in zip(("dweight", "dbias", "dx"), grads, egrads):
+        assert_close(g, e, atol=1e-5 * max(1.0, (inner / 2) ** 0.5) if name != "dx" else 1e-5, what=name)
+
+
 def test_gated_dispatcher_and_errors():
     import gridnet_amd
     from gridnet_amd.backend_cuda import GatedGridnetCudaOp
