@@ -107,19 +107,23 @@ def test_batch_sizes(batch, bs):
     compare(((16, 8, 8), bs, 2, False, "leaky_relu"), batch=batch)
 
 
+@pytest.mark.parametrize("normalize", [False, True], ids=["plain", "normalize"])
+@pytest.mark.parametrize("bs", [8, 4])
 @pytest.mark.parametrize("inner", [16, 32])
-def test_deep_inner_iterations(inner):
+def test_deep_inner_iterations(inner, bs, normalize):
     # small weights keep 32 residual updates tame: with larger ones the 27-term fp32 sums of 32
     # chained iterations leave single entries of dweight a few 1e-6 past the bar
-    shape, bs = (8, 8, 16), 8
+    shape = (8, 8, 16)
     w, b, r = make_params(shape, seed=3)
     w, r = w * 0.25, r * 0.2
     x, gy = make_acts(2, shape, seed=4), make_acts(2, shape, seed=5)
-    y, grads = run_op(w, b, r, x, gy, inner, bs, 1e-5, False, "tanh")
-    ey, eg = oracle(w, b, r, x, gy, inner, bs, 1e-5, False, "tanh")
-    assert_close(y, ey, what="y")
+    y, grads = run_op(w, b, r, x, gy, inner, bs, 1e-5, normalize, "tanh")
+    ey, eg = oracle(w, b, r, x, gy, inner, bs, 1e-5, normalize, "tanh")
+    # with normalize every iteration divides by (std + eps) and takes two window sums more
+    rtol, atol = (2e-4, 2e-5) if normalize else (RTOL, ATOL)
+    assert_close(y, ey, rtol, atol, what="y")
     for name, g, e in zip(("dweight", "dbias", "dscale", "dx"), grads, eg):
-        assert_close(g, e, what=name)
+        assert_close(g, e, rtol, atol, what=name)
 
 
 def test_empty_batch_returns_a_clone():
