@@ -8,6 +8,7 @@ CPU baseline (the reference-style torch path, timed on this machine's host cores
 """
 
 import argparse
+import dataclasses
 import json
 import os
 import sys
@@ -155,6 +156,9 @@ def main():
                     help="fused: the entry points with the LayerNorm folded into the step kernels "
                          "(the faster of the two on MI355X as measured); steps: one call per step "
                          "and per LayerNorm, as the reference's callers do")
+    ap.add_argument("--normalize", action="store_true",
+                    help="the workload with normalize=True (the reference's default, which its "
+                         "training scripts switch off); op-by-op path")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true",
                     help="skip the HIP graph replay (for runs under a counter-collecting profiler)")
@@ -165,6 +169,8 @@ def main():
     from gridnet_amd.configs import WORKLOADS
 
     wl = WORKLOADS[args.workload]
+    if args.normalize:
+        wl = dataclasses.replace(wl, normalize=True, name=wl.name + " normalize")
     fused = args.path == "fused" and not wl.normalize and wl.inner >= 1
     wall, graph_s, kernel_s = gpu_run(wl, args.steps, args.warmup, fused, not args.no_graph)
     bytes_ = wl.algorithmic_bytes()
@@ -177,7 +183,8 @@ def main():
     traffic = None
     try:
         with open(os.path.join(ROOT, "profiles", "traffic.json")) as fh:
-            traffic = json.load(fh).get(args.workload, {}).get("fused" if fused else "steps", {}).get(dominant)
+            variant = "normalize" if args.normalize else "fused" if fused else "steps"
+            traffic = json.load(fh).get(args.workload, {}).get(variant, {}).get(dominant)
     except OSError:
         pass
     dom_s = kernel_s[dominant]

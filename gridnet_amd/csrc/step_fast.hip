@@ -60,7 +60,8 @@ constexpr int kFwdDepth = 9;  // neighbour rows requested ahead of the arithmeti
 // stencil itself is unchanged; the statistics come from sums the threads keep of their own
 // cells (the halo never changes, its sums are taken once, when the window is committed).
 template <int BS, int CPT, int NSLOT, int ACT, bool LN, bool RES = false, bool NORM = false>
-__global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT)) __attribute__((amdgpu_waves_per_eu(3)))
+__global__ __launch_bounds__((Tile<BS, CPT>::TPS * NSLOT))
+__attribute__((amdgpu_waves_per_eu((NORM && CPT >= 4) ? 2 : 3)))  // NORM at 108 weights: no room at 168 registers
 void step_fwd_fast(
     const float *__restrict__ weight, const float *__restrict__ bias,
     const float *__restrict__ scale, const float *__restrict__ x, float *__restrict__ y, int B, int M,
@@ -471,8 +472,11 @@ template <int BS, int CPT> __host__ __device__ constexpr int bwd_slot_floats(int
 template <int BS, int CPT> __host__ __device__ constexpr int bwd_norm_waves() {
     return Tile<BS, CPT>::TPS >= 64 ? Tile<BS, CPT>::TPS / 64 : 1;
 }
+// ... and three values per owned cell that live as long as the kernel but are touched once per
+// iteration or element (sum of the cell's weights, sum of those whose taps read the halo, D2
+// summed over the batch): in LDS, the register file has no room for them
 template <int BS, int CPT> __host__ __device__ constexpr int bwd_norm_floats(int inner) {
-    return 4 * inner + 12 * bwd_norm_waves<BS, CPT>();
+    return 4 * inner + 12 * bwd_norm_waves<BS, CPT>() + 3 * CPT * Tile<BS, CPT>::TPS;
 }
 // ... and at least the 27 weight planes of the block, which pass through LDS once at set-up
 template <int BS, int CPT, int NSLOT> size_t bwd_lds_bytes(int inner, bool ln = false, bool norm = false) {
@@ -558,8 +562,12 @@ void step_bwd_fast(
     const long cells = (long)M * N * K;
     // NORM: the slot's statistics per iteration and the sums its waves exchange
     constexpr int NW = bwd_norm_waves<BS, CPT>();
-    float *nstat = lds + NSLOT * slot_floats + pl.slot * bwd_norm_floats<BS, CPT>(inner);
+    const int norm_stride = bwd_norm_floats<BS, CPT>(inner);
+    float *nstat = lds + NSLOT * slot_floats + pl.slot * norm_stride;
     float *ncommit = nstat + 4 * inner, *nown = ncommit + 4 * NW, *nrev = nown + 4 * NW;
+    float *wsum_at = nrev + 4 * NW + pl.lane * CPT;  // this thread's: sum of a cell's weights
+    float *wout_at = wsum_at + CPT * TL::TPS;         // of those whose taps read the halo
+    float *d2acc_at = wout_at + CPT * TL::TPS;        // D2 summed over the batch elements
     const int wave_in_slot = TL::TPS >= 64 ? pl.lane / 64 : 0;
     constexpr float inv_count = 1.f / TL::NWIN;
 
@@ -623,18 +631,23 @@ void step_bwd_fast(
                                          : 0.f;
         lds_barrier();  // the windows reuse this memory
     }
-    // NORM: sum of a cell's 27 weights, and of those whose taps read the halo
-    float wsum[CPT], wout[CPT], zero[CPT], d2acc[CPT];
+    // NORM: sum of a cell's 27 weights, and of those whose taps read the halo (only this thread
+    // ever touches its three LDS entries per cell: no barrier needed for them)
+    float zero[CPT];
     if (NORM) {
+        float wsum[CPT], wout[CPT];
 #pragma unroll
         for (int c = 0; c < CPT; ++c) {
-            wsum[c] = wout[c] = zero[c] = d2acc[c] = 0.f;
+            wsum[c] = wout[c] = zero[c] = 0.f;
 #pragma unroll
             for (int t = 0; t < 27; ++t) {
                 wsum[c] += w[t][c];
                 wout[c] += in_block(t, c) ? 0.f : w[t][c];
             }
         }
+        store_cells<CPT>(wsum_at, wsum);
+        store_cells<CPT>(wout_at, wout);
+        store_cells<CPT>(d2acc_at, zero);
     }
     typename Fetch<TL>::Buf pre;
     if (ln_in && pl.slot == 0) {  // gamma and beta of the window, once per workgroup
@@ -785,6 +798,8 @@ void step_bwd_fast(
                     inv = 1.f / (sd + norm_eps);
                     if (pl.lane == 0) *reinterpret_cast<float4 *>(nstat + 4 * it) = make_float4(mean, sd, inv, 0.f);
                     stencil<TL, CPT, kBwdDepth>(win + (it & 1) * TL::WIN, pl.row00, w, zero, u);
+                    float wsum[CPT];
+                    load_cells<CPT>(wsum_at, wsum);
 #pragma unroll
                     for (int c = 0; c < CPT; ++c) u[c] = fmaf(inv, fmaf(-mean, wsum[c], u[c]), bv[c]);
                 } else {
@@ -893,6 +908,8 @@ void step_bwd_fast(
                 // A = sum dn and sum dn * x over the whole window, the halo through its brackets
                 float pa = 0.f, pb = 0.f;
                 if (active) {
+                    float wout[CPT];
+                    load_cells<CPT>(wout_at, wout);
 #pragma unroll
                     for (int c = 0; c < CPT; ++c) {
                         pa += fmaf(dlt[c], wout[c], dn[c]);
@@ -934,7 +951,13 @@ void step_bwd_fast(
             g_done[c] = g[c];
             d_done[c] = dsum[c];
             if (RES) gin_done[c] = gin[c];
-            if (NORM && active) d2acc[c] += d2[c];
+        }
+        if (NORM && active) {
+            float d2acc[CPT];
+            load_cells<CPT>(d2acc_at, d2acc);
+#pragma unroll
+            for (int c = 0; c < CPT; ++c) d2acc[c] += d2[c];
+            store_cells<CPT>(d2acc_at, d2acc);
         }
         if (NORM) {
             q_done = q_sum;
@@ -969,11 +992,27 @@ void step_bwd_fast(
                 reduce(dgam[c]);
                 reduce(dbet[c]);
             }
-            if (NORM) reduce(d2acc[c]);
+        }
+        if (NORM) {  // D2 of the other slots: their entries lie one slot's stride further each
+            lds_barrier();
+            if (pl.slot == 0) {
+                float d2acc[CPT];
+                load_cells<CPT>(d2acc_at, d2acc);
+#pragma unroll
+                for (int q = 1; q < NSLOT; ++q) {
+                    float more[CPT];
+                    load_cells<CPT>(d2acc_at + q * norm_stride, more);
+#pragma unroll
+                    for (int c = 0; c < CPT; ++c) d2acc[c] += more[c];
+                }
+                store_cells<CPT>(d2acc_at, d2acc);
+            }
         }
         if (pl.slot != 0) return;
     }
     if (NORM) {  // the taps that read the halo: x_h D1 was added per element, D2 is still owed
+        float d2acc[CPT];
+        load_cells<CPT>(d2acc_at, d2acc);
 #pragma unroll
         for (int t = 0; t < 27; ++t)
 #pragma unroll
