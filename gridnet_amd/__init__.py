@@ -107,7 +107,8 @@ class Gridnet(nn.Module):
                             self.activation)
 
 
-from .network import GridnetBody  # noqa: E402
+from .network import FusedBodyOp, GridnetBody, fused_body  # noqa: E402
 
 __all__ = ["gridnet_step", "gated_gridnet_step", "Gridnet", "GatedGridnet", "GridnetCudaOp",
-           "GatedGridnetCudaOp", "GridLayerNorm", "grid_layer_norm", "GridnetBody"]
+           "GatedGridnetCudaOp", "GridLayerNorm", "grid_layer_norm", "GridnetBody", "FusedBodyOp",
+           "fused_body"]

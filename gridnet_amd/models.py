@@ -21,6 +21,7 @@ import torch.nn as nn
 
 from . import GatedGridnet, Gridnet
 from .layernorm import GridLayerNorm
+from .network import fused_body
 
 
 class Readout(nn.Module):
@@ -44,8 +45,12 @@ class MnistGridModel(nn.Module):
 
     def __init__(self, inner_iters: int, outer_iters: int, init_scale: float,
                  residual_scale: float, activation: str, gated: bool, remember_bias: float,
-                 device):
+                 device, fused_body: bool = False):
         super().__init__()
+        # not in the reference: run the loop as one autograd node on the fused entry points
+        if fused_body and gated:
+            raise ValueError("the fused body covers the plain (not gated) network only")
+        self.fused_body = fused_body
         self.outer_iters = outer_iters
         self.device = device
         self.init_in = nn.Parameter(torch.randn(32, 32, 32, device=device))
@@ -69,6 +74,8 @@ class MnistGridModel(nn.Module):
 
     def forward(self, batch: torch.Tensor) -> torch.Tensor:
         h = self.embed(batch)
+        if self.fused_body:
+            return self.readout(fused_body(h, self.network, self.norm, self.outer_iters))
         for _ in range(self.outer_iters):
             h = self.norm(self.network(h))
         return self.readout(h)
@@ -79,9 +86,13 @@ class ImageNetGridModel(nn.Module):
 
     def __init__(self, *, inner_iters: int, outer_iters: int, outer_residual: bool,
                  init_scale: float, residual_scale: float, emb_channels: int, grid_size: int,
-                 activation: str, separate_params: bool, device):
+                 activation: str, separate_params: bool, device, fused_body: bool = False):
         super().__init__()
         assert 256 % grid_size == 0
+        # not in the reference: run the loop as one autograd node on the fused entry points
+        if fused_body and separate_params:
+            raise ValueError("the fused body shares its parameters between the outer iterations")
+        self.fused_body = fused_body
         self.outer_iters = outer_iters
         self.outer_residual = outer_residual
         self.emb_channels = emb_channels
@@ -110,6 +121,9 @@ class ImageNetGridModel(nn.Module):
 
     def forward(self, images: torch.Tensor) -> torch.Tensor:
         h = self.embed(images)
+        if self.fused_body:
+            return self.readout(fused_body(h, self.network, self.norm, self.outer_iters,
+                                           self.outer_residual))
         for i in range(self.outer_iters):
             net = self.networks[i] if self.separate_params else self.network
             if self.outer_residual:

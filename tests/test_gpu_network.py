@@ -197,3 +197,62 @@ def test_autograd_body_matches_runner():
     assert_close(body.network.weight.grad, grads[0], what="dweight")
     assert_close(body.norm.weight.grad, grads[3], what="dgamma")
     assert_close(x.grad, grads[5], what="dx0")
+
+
+@pytest.mark.parametrize("outer_residual", [False, True], ids=["plain", "outer_residual"])
+@pytest.mark.parametrize("bs", [8, 4])
+def test_fused_autograd_body_matches_op_by_op_body(bs, outer_residual):
+    """GridnetBody(fused=True): the loop as one autograd node on the fused entry points, against
+    the same module looping over the step and LayerNorm ops; two forwards are outstanding before
+    the first backward runs (every call owns its buffers)."""
+    from gridnet_amd import GridnetBody
+
+    shape, inner, outer, batch = (16, 16, 8), 2, 3, 5
+    print(f"fused autograd body bs={bs} outer_residual={outer_residual}", flush=True)
+    torch.manual_seed(5)
+    bodies = [GridnetBody(shape, inner, outer, bs, DEV, "silu", outer_residual=outer_residual, fused=f)
+              for f in (False, True)]
+    with torch.no_grad():
+        for p in bodies[0].parameters():
+            p.add_(0.1 * torch.randn_like(p))
+    bodies[1].load_state_dict(bodies[0].state_dict())
+    xs = [torch.randn(batch, *shape, device=DEV) for _ in range(2)]
+    gys = [torch.randn(batch, *shape, device=DEV) for _ in range(2)]
+    results = []
+    for body in bodies:
+        leaves = [x.clone().requires_grad_(True) for x in xs]
+        outs = [body(leaf) for leaf in leaves]          # both forwards first
+        for out, gy in zip(outs, gys):
+            out.backward(gy)                            # gradients of the parameters add up
+        results.append([o.detach() for o in outs] + [leaf.grad for leaf in leaves] +
+                       [p.grad for p in body.parameters()])
+    names = ["y0", "y1", "dx0", "dx1"] + [n for n, _ in bodies[0].named_parameters()]
+    for name, want, got in zip(names, *results):
+        assert_close(got, want, atol=1e-5 if name[0] in "yd" and "." not in name else 4e-5, what=name)
+    with torch.no_grad():                               # no graph: nothing is kept for a backward
+        assert_close(bodies[1](xs[0]), results[0][0], what="y without grad")
+
+
+def test_models_with_the_fused_body_match_the_reference_loop():
+    from gridnet_amd.models import ImageNetGridModel, MnistGridModel
+
+    torch.manual_seed(6)
+    dev = torch.device(DEV)
+    print("models with fused_body", flush=True)
+    pairs = []
+    a = MnistGridModel(2, 2, 1.0, 1.0, "leaky_relu", False, 0.0, dev)
+    b = MnistGridModel(2, 2, 1.0, 1.0, "leaky_relu", False, 0.0, dev, fused_body=True)
+    pairs.append((a, b, torch.rand(3, 1, 28, 28, device=dev)))
+    kw = dict(inner_iters=2, outer_iters=2, outer_residual=True, init_scale=1.0, residual_scale=0.5,
+              emb_channels=4, grid_size=16, activation="silu", separate_params=False, device=dev)
+    pairs.append((ImageNetGridModel(**kw), ImageNetGridModel(fused_body=True, **kw),
+                  torch.randn(2, 3, 256, 256, device=dev)))
+    for plain, fused, batch in pairs:
+        fused.load_state_dict(plain.state_dict())
+        for m in (plain, fused):
+            m(batch).square().mean().backward()
+        torch.testing.assert_close(fused(batch), plain(batch), rtol=1e-4, atol=1e-5)
+        for (name, p), q in zip(plain.named_parameters(), fused.parameters()):
+            torch.testing.assert_close(q.grad, p.grad, rtol=1e-3, atol=1e-5, msg=lambda m, n=name: f"{n}: {m}")
+    with pytest.raises(ValueError):
+        MnistGridModel(2, 2, 1.0, 1.0, "tanh", True, 0.0, dev, fused_body=True)
