@@ -263,18 +263,23 @@ __device__ __forceinline__ float partner_lane(float v) {
 }
 
 // LN, RES: the variants with the LayerNorm of the network body folded in, as in step_fwd_fast.
-template <int ACT, bool LN, bool RES = false>
-__global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(3)))
+// NORM: per-window normalisation, as in step_fwd_fast (running sums, unchanged stencil).
+template <int ACT, bool LN, bool RES = false, bool NORM = false>
+__global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(NORM ? 2 : 3)))
 void step_fwd_split(
     const float *__restrict__ weight, const float *__restrict__ bias,
     const float *__restrict__ scale, const float *__restrict__ x, float *__restrict__ y, int B, int M,
-    int N, int K, int inner, int nblk, int nchunk, int chunk_len, LnFold ln) {
+    int N, int K, int inner, int nblk, int nchunk, int chunk_len, LnFold ln, float norm_eps) {
     using TL = Tile<8, 4>;
     using SW = SplitWin;
     using FX = Fetch<TL>;
-    // two copies of the window; then, for the folded LayerNorm, gamma and beta laid out alike
-    __shared__ __attribute__((aligned(16))) float lds[(LN ? 4 : 2) * SW::COPY];
+    static_assert(!(NORM && (LN || RES)), "the folded LayerNorm comes without normalisation");
+    // two copies of the window; then, for the folded LayerNorm, gamma and beta laid out alike;
+    // for NORM, per wave the four sums taken at commit and, twice, the two of the owned cells
+    __shared__ __attribute__((aligned(16))) float lds[(LN ? 4 : 2) * SW::COPY + (NORM ? 16 : 0)];
     float *gwin = lds + 2 * SW::COPY, *bwin = gwin + SW::COPY;
+    float *sums_at_commit = lds + 2 * SW::COPY, *own_sums = sums_at_commit + 8;  // NORM: [2][4], [2][2][2]
+    const int wave = threadIdx.x >> 6;
     const bool ln_in = LN && ln.x_stats != nullptr;  // x is the raw output of the step before
 
     int blk, chunk;
@@ -324,10 +329,22 @@ void step_fwd_split(
             rv[r] = second ? rt[3 - r] : rt[r];
         }
     }
+    float wsum[4];  // NORM: sum of the 27 weights of every owned cell
+    if (NORM) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            wsum[r] = 0.f;
+#pragma unroll
+            for (int t = 0; t < 27; ++t) wsum[r] += w[t][r];
+        }
+    }
     // A fetched element goes into `copies` window copies at `to`; with `fold` the LayerNorm of
     // the producer is applied on the way: (v - mean) * rstd * gamma + beta, gamma and beta from
     // their own windows; entries outside the grid stay zero.
+    float part[4];  // NORM: what the last commit added up
     auto commit = [&](float *to, int copies, const typename FX::Buf &v, bool fold, float mean, float rstd) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) part[q] = 0.f;
 #pragma unroll
         for (int e = 0; e < FX::RPT; ++e)
             if (fx.loff[e] >= 0) {
@@ -346,6 +363,16 @@ void step_fwd_split(
                 if (!(fx.ok[e] && fx.edge_ok[e])) end = 0.f;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) c[r] = fx.ok[e] ? c[r] : 0.f;
+                if (NORM) {  // (sum, sum of squares) of the halo entries and of the block's cells
+                    const int row = (pl.lane + e * TL::TPS) >> 1, wj = row % SW::S, wi = row / SW::S;
+                    const bool halo_row = wi == 0 || wi == SW::S - 1 || wj == 0 || wj == SW::S - 1;
+                    const float s1 = (c[0] + c[1]) + (c[2] + c[3]);
+                    const float s2 = fmaf(c[0], c[0], fmaf(c[1], c[1], fmaf(c[2], c[2], c[3] * c[3])));
+                    part[0] += end + (halo_row ? s1 : 0.f);
+                    part[1] += fmaf(end, end, halo_row ? s2 : 0.f);
+                    part[2] += halo_row ? 0.f : s1;
+                    part[3] += halo_row ? 0.f : s2;
+                }
                 for (int copy = 0; copy < copies; ++copy) {
                     *reinterpret_cast<float4 *>(to + copy * SW::COPY + cen_at[e]) =
                         make_float4(c[0], c[1], c[2], c[3]);
@@ -385,6 +412,13 @@ void step_fwd_split(
     for (int s = s0; s < s1; ++s) {
         take_turns(s);
         commit(lds, 2, pre, ln_in, pre_mean, pre_rstd);
+        if (NORM) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) part[q] = slot_wave_sum<64>(part[q]);
+            if ((threadIdx.x & 63) == 0)
+                *reinterpret_cast<float4 *>(sums_at_commit + wave * 4) =
+                    make_float4(part[0], part[1], part[2], part[3]);
+        }
         lds_barrier();
         if (done_s >= 0) store_result(done_s, done);
         if (s + 1 < s1) fetch_element(s + 1);  // next element, in flight
@@ -392,6 +426,12 @@ void step_fwd_split(
         {
             const float4 q = *reinterpret_cast<const float4 *>(lds + own);
             cur[0] = q.x; cur[1] = q.y; cur[2] = q.z; cur[3] = q.w;
+        }
+        float halo1 = 0.f, halo2 = 0.f, own1 = 0.f, own2 = 0.f;  // NORM: sums over the window
+        if (NORM) {
+            const float4 a4 = *reinterpret_cast<const float4 *>(sums_at_commit);
+            const float4 b4 = *reinterpret_cast<const float4 *>(sums_at_commit + 4);
+            halo1 = a4.x + b4.x; halo2 = a4.y + b4.y; own1 = a4.z + b4.z; own2 = a4.w + b4.w;
         }
         if (RES) {  // the raw input of the owned cells, in register order like `cur`
             float rt[4];
@@ -405,8 +445,19 @@ void step_fwd_split(
         for (int it = 0; it < inner; ++it) {
             const float *from = lds + (it & 1) * SW::COPY;
             float u[4];
+            float nmean = 0.f, ninv = 1.f;
+            if (NORM) {
+                if (it > 0) {
+                    const float4 o4 = *reinterpret_cast<const float4 *>(own_sums + (it & 1) * 4);
+                    own1 = o4.x + o4.z;
+                    own2 = o4.y + o4.w;
+                }
+                nmean = (halo1 + own1) * (1.f / 1000);
+                const float var = fmaxf(fmaf(-nmean, nmean, (halo2 + own2) * (1.f / 1000)), 0.f);
+                ninv = 1.f / (sqrtf(var) + norm_eps);
+            }
 #pragma unroll
-            for (int r = 0; r < 4; ++r) u[r] = bv[r];
+            for (int r = 0; r < 4; ++r) u[r] = NORM ? 0.f : bv[r];
 #pragma unroll
             for (int a = 0; a < 3; ++a)
 #pragma unroll
@@ -423,10 +474,21 @@ void step_fwd_split(
                         for (int r = 0; r < 4; ++r)
                             u[r] = fmaf(w[a * 9 + b * 3 + cc][r], v[r + cc], u[r]);
                 }
+            if (NORM) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) u[r] = fmaf(ninv, fmaf(-nmean, wsum[r], u[r]), bv[r]);
+            }
 #pragma unroll
             for (int r = 0; r < 4; ++r) cur[r] = fmaf(rv[r], Act<ACT, float>::f(u[r]), cur[r]);
             *reinterpret_cast<float4 *>(lds + ((it + 1) & 1) * SW::COPY + own) =
                 make_float4(cur[0], cur[1], cur[2], cur[3]);
+            if (NORM && it + 1 < inner) {  // the owned cells' part of the next statistics
+                const float s1 = slot_wave_sum<64>((cur[0] + cur[1]) + (cur[2] + cur[3]));
+                const float s2 = slot_wave_sum<64>(
+                    fmaf(cur[0], cur[0], fmaf(cur[1], cur[1], fmaf(cur[2], cur[2], cur[3] * cur[3]))));
+                if ((threadIdx.x & 63) == 0)
+                    *reinterpret_cast<float2 *>(own_sums + ((it + 1) & 1) * 4 + wave * 2) = make_float2(s1, s2);
+            }
             lds_barrier();
         }
         if (RES) {
@@ -1369,8 +1431,9 @@ int launch_fwd_ln(const StepArgs &a, hipStream_t st) {
                        p.chunk_len, a.ln, (float)a.eps);
     return check_launch("step_fwd_fast");
 }
-template <int ACT, bool LN, bool RES = false> int launch_fwd_split(const StepArgs &a, hipStream_t st) {
-    auto kern = step_fwd_split<ACT, LN, RES>;
+template <int ACT, bool LN, bool RES = false, bool NORM = false>
+int launch_fwd_split(const StepArgs &a, hipStream_t st) {
+    auto kern = step_fwd_split<ACT, LN, RES, NORM>;
     static int per_cu = 0;
     if (per_cu == 0) {
         int n = 0;
@@ -1381,11 +1444,14 @@ template <int ACT, bool LN, bool RES = false> int launch_fwd_split(const StepArg
     hipLaunchKernelGGL(kern, dim3(padded_grid(p.nblk, p.nchunk)), dim3(128), 0, st,
                        (const float *)a.weight, (const float *)a.bias, (const float *)a.scale,
                        (const float *)a.x, (float *)a.y, a.B, a.M, a.N, a.K, a.inner, p.nblk, p.nchunk,
-                       p.chunk_len, a.ln);
+                       p.chunk_len, a.ln, (float)a.eps);
     return check_launch("step_fwd_split");
 }
 template <int BS, int CPT, int NSLOT, int ACT> int launch_fwd(const StepArgs &a, hipStream_t st) {
-    if (a.normalize) return launch_fwd_ln<BS, CPT, NSLOT, ACT, false, false, true>(a, st);
+    if (a.normalize) {
+        if (BS == 8) return launch_fwd_split<ACT, false, false, true>(a, st);
+        return launch_fwd_ln<BS, CPT, NSLOT, ACT, false, false, true>(a, st);
+    }
     if (a.ln.gamma && a.ln.residual) {
         if (BS == 8) return launch_fwd_split<ACT, true, true>(a, st);
         return launch_fwd_ln<BS, CPT, NSLOT, ACT, true, true>(a, st);
