@@ -57,6 +57,21 @@ def test_host_only_entry_points():
     assert rc == 1 and "grid too large" in native.last_error()
     rc = native.lib.gridnet_hip_forward(0, None, 8, 8, 8, 8, 1, 424, 424, 424, 1, 8, 1e-5, 0, 0, None)
     assert rc == 1 and "null input pointer" in native.last_error()
+    # backward workspaces: one activation tensor (D) for the plain step, two floats per block and
+    # batch element more with normalize, two tensors (D0, D1) for the gated step; none in fp64
+    act = 32 * 64 ** 3 * 4
+    assert native.lib.gridnet_hip_backward_workspace_bytes(0, 32, 64, 64, 64, 4, 8, 0) == act
+    assert native.lib.gridnet_hip_backward_workspace_bytes(0, 32, 64, 64, 64, 4, 8, 1) == act + 32 * 512 * 8
+    assert native.lib.gridnet_hip_backward_workspace_bytes(1, 32, 64, 64, 64, 4, 8, 0) == 0
+    assert native.lib.gridnet_hip_backward_gated_workspace_bytes(0, 32, 64, 64, 64, 4, 8) == 2 * act
+    assert native.lib.gridnet_hip_backward_gated_workspace_bytes(1, 32, 64, 64, 64, 4, 8) == 0
+    # the history of more than 21 inner iterations does not fit the LDS at 8^3 blocks: generic kernels
+    assert native.lib.gridnet_hip_backward_gated_workspace_bytes(0, 32, 64, 64, 64, 22, 8) == 0
+    rc = native.lib.gridnet_hip_backward_gated(0, 8, 8, 8, 8, 8, 8, 8, 2, 8, 8, 8, 2, 8, 0, 0, None, 0, None)
+    assert rc == 4 and "workspace" in native.last_error()
+    rc = native.lib.gridnet_hip_backward(0, 8, 8, 8, 8, 8, 8, 8, 8, 8, 2, 8, 8, 8, 2, 8, 1e-5, 1, 0, 0,
+                                         None, 0, None)
+    assert rc == 4 and "workspace" in native.last_error()
     assert native.lib.gridnet_hip_layernorm_workspace_bytes(0, 32, 64 ** 3) == (32 * 64 * 2 + 64) * 4
     rc = native.lib.gridnet_hip_layernorm_forward(0, 8, 8, 8, 8, 8, 8, 4, 4096, 1e-5, None, 0, None)
     assert rc == 4 and "workspace" in native.last_error()
