@@ -75,7 +75,7 @@ struct LayerNormArgs {
 int step_forward_generic(const StepArgs &a, hipStream_t st);
 int step_backward_generic(const StepArgs &a, hipStream_t st);
 
-// step_fast.hip: fp32, normalize=false; return -1 when the problem is outside what they cover
+// step_fast.hip: fp32, block sizes 4 and 8, normalize on or off (off only with the folded LayerNorm)
 bool step_fast_supports(const StepArgs &a, bool backward);
 size_t step_fast_backward_workspace(const StepArgs &a);
 int step_forward_fast(const StepArgs &a, hipStream_t st);

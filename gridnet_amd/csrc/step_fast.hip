@@ -1,5 +1,7 @@
-// Tuned fp32 kernels for the block-local update with normalize=false (every configuration the
-// reference's training scripts use: gridnet/scripts/train_mnist.py:51, train_imagenet.py:50).
+// Tuned fp32 kernels for the block-local update.  Written for normalize=false (every
+// configuration the reference's training scripts use: gridnet/scripts/train_mnist.py:51,
+// train_imagenet.py:50); the NORM variants add the per-window normalisation of the reference's
+// default on top (see step_fwd_fast and step_bwd_fast).
 //
 // Mapping.  A "slot" is the group of threads that advances ONE (spatial block, batch element)
 // pair: bs*bs*(bs/CPT) threads, each owning CPT consecutive cells of a K-row together with

@@ -1,6 +1,7 @@
 // Generic block-local update kernels: one thread per cell, any dtype (fp32/fp64), any
 // activation, optional per-window normalisation, up to 32 inner iterations in backward.
-// This is the coverage path; the tuned fp32 kernels for normalize=false are separate.
+// This is the coverage path (fp64, and fp32 problems the tuned kernels decline); the tuned fp32
+// kernels are separate (step_fast.hip).
 //
 // Work decomposition: one workgroup owns one spatial block (bs^3 threads) and walks a chunk
 // of batch elements with the block's 27 weights, bias and scale held in registers, so the
