@@ -245,11 +245,15 @@ template <typename TL, int NT = TL::TPS> struct Fetch {  // NT: threads of a slo
                 }
             }
     }
-    // The plain commit, which also adds up what it writes: (sum, sum of squares) of the halo
-    // entries in part[0..1], of the block's own cells in part[2..3] (entries outside the grid are
-    // zeros and add nothing).  For the per-window normalisation.
+    // The commit for the per-window normalisation: every entry is written MINUS `shift` (entries
+    // outside the grid, zeros, become -shift) and what is written is added up: (sum, sum of
+    // squares) of the halo entries in part[0..1], of the block's own cells in part[2..3].
+    // Normalising a window does not care about a common shift of its entries; with `shift` a value
+    // from the window itself the sums stay small, and variance = E[x^2] - mean^2 keeps its digits
+    // however far the data sits from zero.
     template <int COPIES = 2>
-    __device__ __forceinline__ void commit_sums(float *win, const Buf &v, float (&part)[4]) const {
+    __device__ __forceinline__ void commit_sums(float *win, const Buf &v, float shift,
+                                                float (&part)[4]) const {
 #pragma unroll
         for (int q = 0; q < 4; ++q) part[q] = 0.f;
 #pragma unroll
@@ -258,20 +262,26 @@ template <typename TL, int NT = TL::TPS> struct Fetch {  // NT: threads of a slo
                 const int row = (lane0 + e * NT) >> 1;
                 const int wj = row % S, wi = row / S;
                 const bool halo_row = wi == 0 || wi == S - 1 || wj == 0 || wj == S - 1;
-                const float end = (ok[e] && edge_ok[e]) ? v[e][HC] : 0.f;
-                float s1 = 0.f, s2 = 0.f;
+                const float end = ((ok[e] && edge_ok[e]) ? v[e][HC] : 0.f) - shift;
+                float c[HC], s1 = 0.f, s2 = 0.f;
 #pragma unroll
                 for (int q = 0; q < HC; ++q) {
-                    const float c = ok[e] ? v[e][q] : 0.f;
-                    s1 += c;
-                    s2 = fmaf(c, c, s2);
+                    c[q] = (ok[e] ? v[e][q] : 0.f) - shift;
+                    s1 += c[q];
+                    s2 = fmaf(c[q], c[q], s2);
                 }
                 part[0] += end + (halo_row ? s1 : 0.f);
                 part[1] += fmaf(end, end, halo_row ? s2 : 0.f);
                 part[2] += halo_row ? 0.f : s1;
                 part[3] += halo_row ? 0.f : s2;
+#pragma unroll
+                for (int copy = 0; copy < COPIES; ++copy) {
+                    float *row_at = win + copy * TL::WIN + loff[e];
+                    row_at[hi[e] ? HC : 0] = end;
+#pragma unroll
+                    for (int q = 0; q < HC; ++q) row_at[q + (hi[e] ? 0 : 1)] = c[q];
+                }
             }
-        commit<COPIES>(win, v);
     }
     // The same, with the LayerNorm of the producer applied on the way in: an entry becomes
     // (v - mean) * rstd * gamma + beta; entries outside the grid stay zero.  gamma and beta of a

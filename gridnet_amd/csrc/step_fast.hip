@@ -121,12 +121,17 @@ void step_fwd_fast(
 
     const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
     float pre_mean = 0.f, pre_rstd = 1.f;  // LayerNorm statistics of the element in `pre`
+    // NORM: the window is kept minus one of its own values (the block's first cell), see
+    // Fetch::commit_sums; `shift` belongs to the element being iterated, `pre_shift` to `pre`
+    float pre_shift = 0.f, shift = 0.f, done_shift = 0.f;
+    const int first_cell = (pl.p0 * N + pl.q0) * K + pl.r0;
     auto fetch_element = [&](int s) {
         fx.fetch(x + s * cells, pre);
         if (ln_in) {
             pre_mean = load_ahead(ln.x_stats, 2 * s);
             pre_rstd = load_ahead(ln.x_stats, 2 * s + 1);
         }
+        if (NORM) pre_shift = load_ahead(x + s * cells, first_cell);
     };
     if (s0 + pl.slot < s1) fetch_element(s0 + pl.slot);
     // The result of an element is stored one element late, after the next window has been
@@ -141,7 +146,8 @@ void step_fwd_fast(
             if (ln_in) fx.commit_ln(win, pre, affine, pre_mean, pre_rstd);
             else if (NORM) {
                 float part[4];
-                fx.commit_sums(win, pre, part);
+                shift = pre_shift;
+                fx.commit_sums(win, pre, shift, part);
 #pragma unroll
                 for (int q = 0; q < 4; ++q) part[q] = row16_sum(part[q]);
                 if ((pl.lane & 15) == 0)
@@ -150,7 +156,13 @@ void step_fwd_fast(
             } else fx.commit(win, pre);
         }
         lds_barrier();
-        if (done_s >= 0) store_cells<CPT>(y + done_s * cells + pl.gc, done);
+        if (done_s >= 0) {
+            if (NORM) {
+#pragma unroll
+                for (int c = 0; c < CPT; ++c) done[c] += done_shift;
+            }
+            store_cells<CPT>(y + done_s * cells + pl.gc, done);
+        }
         if (s + NSLOT < s1) fetch_element(s + NSLOT);  // next element, in flight
         float cur[CPT], base[CPT], raw[CPT];
         float halo1 = 0.f, halo2 = 0.f, own1 = 0.f, own2 = 0.f;  // NORM: sums of the window
@@ -231,11 +243,18 @@ void step_fwd_fast(
             }
         }
         done_s = active ? s : -1;
+        done_shift = shift;
 #pragma unroll
         for (int c = 0; c < CPT; ++c) done[c] = cur[c];
         if (inner == 0) lds_barrier();  // `cur` was read from the window that is rewritten next
     }
-    if (done_s >= 0) store_cells<CPT>(y + done_s * cells + pl.gc, done);
+    if (done_s >= 0) {
+        if (NORM) {
+#pragma unroll
+            for (int c = 0; c < CPT; ++c) done[c] += done_shift;
+        }
+        store_cells<CPT>(y + done_s * cells + pl.gc, done);
+    }
 }
 
 // ---- forward, 8^3 blocks: the split window ------------------------------------------------
@@ -344,6 +363,10 @@ void step_fwd_split(
     // the producer is applied on the way: (v - mean) * rstd * gamma + beta, gamma and beta from
     // their own windows; entries outside the grid stay zero.
     float part[4];  // NORM: what the last commit added up
+    // NORM: the window is kept minus one of its own values (the block's first cell), see
+    // Fetch::commit_sums; `pre_shift` belongs to `pre`, `shift` to the element being iterated
+    float pre_shift = 0.f, shift = 0.f, done_shift = 0.f;
+    const int first_cell = (pl.p0 * N + pl.q0) * K + pl.r0;
     auto commit = [&](float *to, int copies, const typename FX::Buf &v, bool fold, float mean, float rstd) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) part[q] = 0.f;
@@ -365,7 +388,10 @@ void step_fwd_split(
                 if (!(fx.ok[e] && fx.edge_ok[e])) end = 0.f;
 #pragma unroll
                 for (int r = 0; r < 4; ++r) c[r] = fx.ok[e] ? c[r] : 0.f;
-                if (NORM) {  // (sum, sum of squares) of the halo entries and of the block's cells
+                if (NORM) {  // minus the shift; (sum, sum of squares) of halo entries and block cells
+                    end -= pre_shift;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) c[r] -= pre_shift;
                     const int row = (pl.lane + e * TL::TPS) >> 1, wj = row % SW::S, wi = row / SW::S;
                     const bool halo_row = wi == 0 || wi == SW::S - 1 || wj == 0 || wj == SW::S - 1;
                     const float s1 = (c[0] + c[1]) + (c[2] + c[3]);
@@ -393,7 +419,7 @@ void step_fwd_split(
     auto store_result = [&](int s, const float (&cur)[4]) {
         float out[4];
 #pragma unroll
-        for (int c = 0; c < 4; ++c) out[c] = second ? cur[3 - c] : cur[c];
+        for (int c = 0; c < 4; ++c) out[c] = (second ? cur[3 - c] : cur[c]) + (NORM ? done_shift : 0.f);
         store_cells<4>(y + s * cells + pl.gc, out);
     };
 
@@ -405,6 +431,7 @@ void step_fwd_split(
             pre_mean = load_ahead(ln.x_stats, 2 * s);
             pre_rstd = load_ahead(ln.x_stats, 2 * s + 1);
         }
+        if (NORM) pre_shift = load_ahead(x + s * cells, first_cell);
     };
     if (s0 < s1) fetch_element(s0);
     // The result of an element is stored one element late, after the next window has been
@@ -415,6 +442,7 @@ void step_fwd_split(
         take_turns(s);
         commit(lds, 2, pre, ln_in, pre_mean, pre_rstd);
         if (NORM) {
+            shift = pre_shift;
 #pragma unroll
             for (int q = 0; q < 4; ++q) part[q] = slot_wave_sum<64>(part[q]);
             if ((threadIdx.x & 63) == 0)
@@ -514,6 +542,7 @@ void step_fwd_split(
             }
         }
         done_s = s;
+        done_shift = shift;
 #pragma unroll
         for (int r = 0; r < 4; ++r) done[r] = cur[r];
         if (inner == 0) lds_barrier();  // `cur` was read from the window that is rewritten next
@@ -751,6 +780,11 @@ void step_bwd_fast(
     // the latter again for the element whose results are stored one element late
     float gprev[CPT], gin[CPT], gin_done[CPT];
     const bool through_ln = LN && (!RES || ln.y_raw != nullptr);  // dy passes a LayerNorm on load
+    // NORM: the x window is kept minus one of its own values (the block's first cell), see
+    // Fetch::commit_sums; everything downstream only sees differences of window entries, except
+    // R, which is handed on for the unshifted x (R + shift * Q)
+    float pre_shift = 0.f, shift = 0.f;
+    const int first_cell = (pl.p0 * N + pl.q0) * K + pl.r0;
     auto fetch_element = [&](int s) {
         fx.fetch(x + s * cells, pre);
         load_cells<CPT>(dy + s * cells + pl.gc, gnext);
@@ -766,6 +800,7 @@ void step_bwd_fast(
             nx_mean = load_ahead(ln.x_stats, 2 * s);
             nx_rstd = load_ahead(ln.x_stats, 2 * s + 1);
         }
+        if (NORM) pre_shift = load_ahead(x + s * cells, first_cell);
     };
     // the element just fetched becomes the current one: its gradient (through the LayerNorm
     // backward for LN) and its window
@@ -786,7 +821,8 @@ void step_bwd_fast(
         if (ln_in) fx.commit_ln(win, pre, affine, nx_mean, nx_rstd);
         else if (NORM) {
             float part[4];
-            fx.commit_sums(win, pre, part);
+            shift = pre_shift;
+            fx.commit_sums(win, pre, shift, part);
 #pragma unroll
             for (int q = 0; q < 4; ++q) part[q] = slot_wave_sum<TL::TPS>(part[q]);
             if ((pl.lane & 63 & (TL::TPS - 1)) == 0)
@@ -1025,7 +1061,7 @@ void step_bwd_fast(
         }
         if (NORM) {
             q_done = q_sum;
-            r_done = r_sum;
+            r_done = fmaf(shift, q_sum, r_sum);
         }
         // the x windows are free (the reverse sweep does not read them): commit the next one
         if (s + NSLOT < s1) take_element();

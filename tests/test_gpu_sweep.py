@@ -102,6 +102,36 @@ def test_random_normalized_step_tuned_fp32_against_generic_fp64(seed):
         assert_close(got, want, rtol=2e-4, atol=summed if name != "y" else 2e-5, what=name)
 
 
+@pytest.mark.parametrize("offset", [30.0, -100.0])
+@pytest.mark.parametrize("bs", [8, 4])
+def test_normalized_step_on_inputs_far_from_zero(bs, offset):
+    """Windows whose mean dwarfs their spread (blocks away from the grid's border, whose windows
+    hold no zeros from outside the grid): the tuned kernels take the window statistics from
+    running sums, variance = E[x^2] - mean^2 as in the reference's kernel
+    (src/gridnet_cuda_kernels.cu:164-170), but of a window that is kept minus one of its own
+    values, so the subtraction does not eat the digits (without that shift the forward result
+    was 7e-3 off at an offset of 100 with 4^3 blocks)."""
+    import gridnet_cuda
+
+    shape, batch, inner = (32, 16, 16), 3, 3
+    print(f"normalized far from zero bs={bs} offset={offset}", flush=True)
+    w, b, r = make_params(shape, seed=7500)
+    x, gy = make_acts(batch, shape, seed=7501) + offset, make_acts(batch, shape, seed=7502)
+
+    def call(dtype):
+        tw, tb, tr, tx, tgy = (t.to(device=DEV, dtype=dtype) for t in (w, b, r, x, gy))
+        y = torch.full_like(tx, float("nan"))
+        gridnet_cuda.forward(tw, tb, tr, tx, y, inner, bs, 1e-5, True, "silu")
+        outs = [torch.zeros_like(t) for t in (tw, tb, tr, tx)]
+        gridnet_cuda.backward(tw, tb, tr, tx, tgy, *outs, inner, bs, 1e-5, True, "silu")
+        return [y] + outs
+
+    fast, slow = call(torch.float32), call(torch.float64)
+    for name, got, want in zip(("y", "dweight", "dbias", "dscale", "dx"), fast, slow):
+        # y carries the offset itself: its fp32 representation alone is 4e-6 off at 100
+        assert_close(got, want, rtol=2e-4, atol=5e-5, what=name)
+
+
 def draw_gated(seed):
     rng = random.Random(8000 + seed)
     bs = rng.choice((4, 8))
