@@ -133,3 +133,27 @@ def test_autograd_op_keeps_the_reference_contract():
     empty = torch.zeros(0, 8, 8, 8)
     out = GridnetCudaOp.apply(w, p, p, empty, 1, 8, 1e-5, False, "silu")
     assert out.shape == empty.shape and out.data_ptr() != empty.data_ptr() or out.numel() == 0
+
+
+def test_shim_matches_the_call_sites_in_the_reference_tree():
+    """Where the reference is on disk (this container, not the GPU box): every call of the
+    extension module in gridnet/backend_cuda.py, read as text and parsed, must fit the shim's
+    function of that name -- same number of positional arguments, no keywords."""
+    import ast
+    import os
+
+    import gridnet_cuda
+
+    path = "/root/reference/gridnet/backend_cuda.py"
+    if not os.path.exists(path):
+        pytest.skip("the reference tree is not on this machine")
+    with open(path) as fh:
+        tree = ast.parse(fh.read())
+    calls = [n for n in ast.walk(tree)
+             if isinstance(n, ast.Call) and isinstance(n.func, ast.Attribute)
+             and isinstance(n.func.value, ast.Name) and n.func.value.id == "gridnet_cuda"]
+    assert {c.func.attr for c in calls} == {"forward", "backward", "forward_gated", "backward_gated"}
+    for call in calls:
+        params = inspect.signature(getattr(gridnet_cuda, call.func.attr)).parameters
+        assert not call.keywords, call.func.attr
+        assert len(call.args) == len(params), (call.func.attr, len(call.args), len(params))
