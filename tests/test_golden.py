@@ -43,14 +43,15 @@ def test_oracle_reproduces_fixture_in_fp32():
 
 
 @pytest.mark.gpu
-def test_hip_path_reproduces_fixture():
+@pytest.mark.parametrize("fused", [False, True], ids=["op-by-op", "fused"])
+def test_hip_path_reproduces_fixture(fused):
     from gridnet_amd.runner import BodyRunner
 
     wl, t = c1()
     gold = np.load(FIXTURE)
     d = {k: v.to("cuda:0") for k, v in t.items()}
     run = BodyRunner(d["weight"], d["bias"], d["scale"], d["gamma"], d["beta"], wl.batch, wl.inner,
-                     wl.outer, wl.block_size, wl.activation, wl.normalize)
+                     wl.outer, wl.block_size, wl.activation, wl.normalize, fused=fused)
     y = run.forward(d["x0"]).clone()
     grads = run.backward(d["grad_out"])
     for name, got in zip(NAMES, (y, *grads)):
