@@ -56,3 +56,51 @@ def test_hip_path_reproduces_fixture(fused):
     grads = run.backward(d["grad_out"])
     for name, got in zip(NAMES, (y, *grads)):
         assert_close(got, torch.from_numpy(gold[name]), what=name)
+
+
+# ---- one outer step with normalize=True and one gated step (tests/golden/make_step_fixtures.py)
+STEP_FIXTURES = {
+    "normalize": ("step_normalize.npz", ("weight", "bias", "scale", "x"), ("y", "dweight", "dbias", "dscale", "dx")),
+    "gated": ("step_gated.npz", ("weight", "bias", "x"), ("y", "dweight", "dbias", "dx")),
+}
+
+
+def load_step(kind):
+    name, inputs, outputs = STEP_FIXTURES[kind]
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", name))
+    return gold, inputs, outputs
+
+
+@pytest.mark.parametrize("kind", sorted(STEP_FIXTURES))
+def test_ref_style_oracle_reproduces_step_fixture_in_fp32(kind):
+    """The op-for-op restatement of the reference's torch path, run in fp32 on the CPU, lands on
+    the fixture (which the vectorised oracle wrote in fp64) within the bar."""
+    from oracle.gated import gated_step_ref
+    from oracle.ref_style import gridnet_step_ref
+
+    gold, inputs, outputs = load_step(kind)
+    leaves = [torch.from_numpy(gold[k]).requires_grad_(True) for k in inputs]
+    if kind == "normalize":
+        y = gridnet_step_ref(*leaves, 3, 4, 1e-5, True, "silu")
+    else:
+        y = gated_step_ref(*leaves, 3, 4, "tanh")
+    grads = torch.autograd.grad(y, leaves, torch.from_numpy(gold["grad_out"]))
+    for name, got in zip(outputs, (y, *grads)):
+        assert_close(got, torch.from_numpy(gold[name]), rtol=2e-4, atol=2e-5, what=f"{kind} {name}")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("kind", sorted(STEP_FIXTURES))
+def test_hip_path_reproduces_step_fixture(kind):
+    from gridnet_amd.backend_cuda import GatedGridnetCudaOp, GridnetCudaOp
+
+    gold, inputs, outputs = load_step(kind)
+    leaves = [torch.from_numpy(gold[k]).to("cuda:0").requires_grad_(True) for k in inputs]
+    if kind == "normalize":
+        y = GridnetCudaOp.apply(*leaves, 3, 4, 1e-5, True, "silu")
+    else:
+        y = GatedGridnetCudaOp.apply(*leaves, 3, 4, "tanh")
+    grads = torch.autograd.grad(y, leaves, torch.from_numpy(gold["grad_out"]).to("cuda:0"))
+    for name, got in zip(outputs, (y, *grads)):
+        assert_close(got, torch.from_numpy(gold[name]), rtol=2e-4 if kind == "normalize" else 1e-4,
+                     atol=2e-5 if kind == "normalize" else 1e-5, what=f"{kind} {name}")
