@@ -256,3 +256,46 @@ def test_models_with_the_fused_body_match_the_reference_loop():
             torch.testing.assert_close(q.grad, p.grad, rtol=1e-3, atol=1e-5, msg=lambda m, n=name: f"{n}: {m}")
     with pytest.raises(ValueError):
         MnistGridModel(2, 2, 1.0, 1.0, "tanh", True, 0.0, dev, fused_body=True)
+
+
+def test_two_streams_in_flight_do_not_disturb_each_other():
+    """The library keeps no state between calls and launches on the stream it is given: two
+    chains enqueued alternately on two streams (their kernels free to overlap on the device)
+    give what each gives alone."""
+    from gridnet_amd.configs import WORKLOADS, make_inputs
+    from gridnet_amd.runner import BodyRunner
+
+    wl = dataclasses.replace(WORKLOADS["C3"], grid=32, batch=6, outer=3)
+    print("two streams", flush=True)
+    inputs = [make_inputs(wl, seed=s) for s in (0, 1)]
+    dev = torch.device(DEV)
+
+    def build(t, fused):
+        d = {k: v.to(dev) for k, v in t.items()}
+        return BodyRunner(d["weight"], d["bias"], d["scale"], d["gamma"], d["beta"], wl.batch, wl.inner,
+                          wl.outer, wl.block_size, "silu", backward=True, fused=fused), d
+
+    alone = []
+    for t, fused in zip(inputs, (True, False)):
+        run, d = build(t, fused)
+        y = run.forward(d["x0"]).clone()
+        alone.append([y] + [g.clone() for g in run.backward(d["grad_out"])])
+    torch.cuda.synchronize()
+
+    runs = [build(t, fused) for t, fused in zip(inputs, (True, False))]
+    streams = [torch.cuda.Stream(device=dev) for _ in runs]
+    for st in streams:
+        st.wait_stream(torch.cuda.current_stream(dev))
+    outs = [None, None]
+    for rep in range(3):  # several rounds, so that the two really are in flight together
+        for i, ((run, d), st) in enumerate(zip(runs, streams)):
+            with torch.cuda.stream(st):
+                y = run.forward(d["x0"])
+                outs[i] = [y] + list(run.backward(d["grad_out"]))
+    torch.cuda.synchronize()
+    for i in range(2):
+        for j, (got, want) in enumerate(zip(outs[i], alone[i])):
+            if j in (0, 6):  # y and dx0: no atomics anywhere, bit for bit the same
+                assert torch.equal(got, want), f"stream {i} output {j}"
+            else:  # 64 blocks < CUs: the batch is split over workgroups, parameter gradients by atomics
+                assert_close(got, want, atol=4e-5, what=f"stream {i} output {j}")
