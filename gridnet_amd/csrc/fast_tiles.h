@@ -70,6 +70,34 @@ template <int TPS> __device__ __forceinline__ float slot_wave_sum(float v) {
     return (r0 + r1) + (r2 + r3);
 }
 
+// (mean, M2 about that mean) of the cells that the lanes of a slot in this wave hold, from the
+// same pair per 16-lane row (each over `row_cells` cells): the rows' means are averaged and the
+// M2 combined with the exact pairwise formula, M2 = sum M2_r + row_cells sum (mean_r - mean)^2.
+// Every lane of the slot gets the same pair.  TPS as for slot_wave_sum.
+template <int TPS>
+__device__ __forceinline__ void slot_wave_moments(float row_mean, float row_m2, int row_cells, float &mean,
+                                                  float &m2) {
+    static_assert(TPS == 32 || TPS % 64 == 0, "slots are half waves or whole waves");
+    float m[4], q[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        m[r] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(row_mean), 16 * r));
+        q[r] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(row_m2), 16 * r));
+    }
+    if (TPS == 32) {
+        const bool upper = (threadIdx.x & 32) != 0;
+        const float a = upper ? m[2] : m[0], b = upper ? m[3] : m[1];
+        mean = 0.5f * (a + b);
+        m2 = (upper ? q[2] + q[3] : q[0] + q[1]) + row_cells * ((a - mean) * (a - mean) + (b - mean) * (b - mean));
+    } else {
+        mean = 0.25f * ((m[0] + m[1]) + (m[2] + m[3]));
+        float dev = 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) dev = fmaf(m[r] - mean, m[r] - mean, dev);
+        m2 = ((q[0] + q[1]) + (q[2] + q[3])) + row_cells * dev;
+    }
+}
+
 // Load p[i], i the same for the whole wave, as a VECTOR memory load.  Left alone the compiler
 // makes it a scalar load; those return out of order and share their counter with LDS, so one
 // that is still on its way stalls the next LDS access for a whole trip to memory -- and the

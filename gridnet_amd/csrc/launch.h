@@ -16,8 +16,8 @@ namespace gridnet {
 struct LnFold {
     const float *gamma, *beta;  // [M,N,K]
     const float *x_stats;       // [B,2]: LayerNorm applied to x on load; null: x is used as is
-    float *y_part;              // forward: partial (mean, M2) of the output, one pair per 16-lane
-                                // group, [B, nblk, groups, 2]
+    float *y_part;              // forward: partial (mean, M2) of the output, one pair per wave
+                                // (per slot, for half-wave slots): [B, nblk, parts, 2]
     // backward: the incoming gradient is with respect to LayerNorm(y_raw)
     const float *y_raw;         // [B,M,N,K] this step's forward output before its LayerNorm
     const float *y_stats;       // [B,2]

@@ -236,10 +236,14 @@ void step_fwd_fast(
 #pragma unroll
             for (int c = 0; c < CPT; ++c) m2 = fmaf(cur[c] - mean, cur[c] - mean, m2);
             m2 = row16_sum(m2);
-            if ((pl.lane & 15) == 0) {
-                float *to = ln.y_part + (((long)s * nblk + blk) * (TL::TPS / 16) + pl.lane / 16) * 2;
-                to[0] = mean;
-                to[1] = m2;
+            // one pair per wave of the slot (per slot, for half-wave slots)
+            constexpr int PARTS = TL::TPS >= 64 ? TL::TPS / 64 : 1;
+            float wave_mean, wave_m2;
+            slot_wave_moments<TL::TPS>(mean, m2, 16 * CPT, wave_mean, wave_m2);
+            if ((pl.lane & (TL::TPS >= 64 ? 63 : 31)) == 0) {
+                float *to = ln.y_part + (((long)s * nblk + blk) * PARTS + (TL::TPS >= 64 ? pl.lane / 64 : 0)) * 2;
+                to[0] = wave_mean;
+                to[1] = wave_m2;
             }
         }
         done_s = active ? s : -1;
@@ -535,10 +539,12 @@ void step_fwd_split(
 #pragma unroll
             for (int r = 0; r < 4; ++r) m2 = fmaf(cur[r] - mean, cur[r] - mean, m2);
             m2 = row16_sum(m2);
-            if ((pl.lane & 15) == 0) {
-                float *to = ln.y_part + (((long)s * nblk + blk) * (TL::TPS / 16) + pl.lane / 16) * 2;
-                to[0] = mean;
-                to[1] = m2;
+            float wave_mean, wave_m2;  // one pair per wave
+            slot_wave_moments<128>(mean, m2, 64, wave_mean, wave_m2);
+            if ((pl.lane & 63) == 0) {
+                float *to = ln.y_part + (((long)s * nblk + blk) * 2 + pl.lane / 64) * 2;
+                to[0] = wave_mean;
+                to[1] = wave_m2;
             }
         }
         done_s = s;
@@ -1347,12 +1353,15 @@ void step_bwd_cross(
                         t1 += a;
                         t2 = fmaf(a, (xr[e][c] - xmean[e]) * xrstd[e], t2);
                     }
-                    t1 = row16_sum(t1);  // the row threads are whole 16-lane groups
-                    t2 = row16_sum(t2);
-                    if ((lane & 15) == 0 && s < s1) {
-                        float *to = ln.x_part + (((long)s * nblk + blk) * (FS / 16) + lane / 16) * 2;
-                        to[0] = t1;
-                        to[1] = t2;
+                    // one pair per (element, block): the row threads are 16 lanes (bs=4), or the
+                    // whole first wave of the slot (bs=8)
+                    static_assert(FS == 16 || (FS == 64 && TPS % 64 == 0), "row threads fill a row or a wave");
+                    const float w1 = FS == 64 ? slot_wave_sum<64>(t1) : row16_sum(t1);
+                    const float w2 = FS == 64 ? slot_wave_sum<64>(t2) : row16_sum(t2);
+                    if (lane == 0 && s < s1) {
+                        float *to = ln.x_part + ((long)s * nblk + blk) * 2;
+                        to[0] = w1;
+                        to[1] = w2;
                     }
                 }
             }
@@ -1620,11 +1629,15 @@ int gated_cross_launch(const StepArgs &a, const float *dsum, int nchunk, int chu
     return check_launch("step_bwd_cross (gated)");
 }
 
+// one pair per wave of a slot, or per slot where a slot is half a wave
 int step_fast_forward_parts(int block_size) {
-    return block_size == 8 ? Tile<8, kFwdCpt8>::TPS / 16 : Tile<4, kFwdCpt4>::TPS / 16;
+    const int tps = block_size == 8 ? Tile<8, kFwdCpt8>::TPS : Tile<4, kFwdCpt4>::TPS;
+    return tps >= 64 ? tps / 64 : 1;
 }
-int step_fast_forward_part_count(int block_size) { return 16 * (block_size == 8 ? kFwdCpt8 : kFwdCpt4); }
-int step_fast_backward_parts(int block_size) { return block_size * block_size / 16; }
+int step_fast_forward_part_count(int block_size) {
+    return block_size * block_size * block_size / step_fast_forward_parts(block_size);
+}
+int step_fast_backward_parts(int) { return 1; }
 
 bool step_fast_supports(const StepArgs &a, bool backward) {
     if (a.dtype != GRIDNET_F32) return false;
