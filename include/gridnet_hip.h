@@ -14,6 +14,10 @@
  *   - A tensor may start at any address that is a multiple of its element size (for example
  *     a view one element into a larger buffer), as with the reference's element-wise
  *     accessors (src/gridnet_cuda_kernels.cu:103-107); the workspace likewise.
+ *   - Sizes: the cells of one sample are indexed with 32 bits, so 27*M*N*K (54*M*N*K for
+ *     the gated op) must stay below 2^31; samples are indexed with 64 bits, so B*M*N*K may
+ *     exceed 2^31 (the reference's 32-bit accessors, src/gridnet_cuda_kernels.cu:103-107,
+ *     stop there).
  *   - Return value 0 = enqueued.  Non-zero = nothing was enqueued; the message is
  *     available from gridnet_hip_last_error() on the calling thread.
  */
