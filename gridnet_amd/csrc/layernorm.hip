@@ -277,25 +277,31 @@ __global__ __launch_bounds__(kLnThreads) void ln_bwd_apply(
 // The step kernels leave per-group partial results; these small kernels turn them into the
 // per-sample numbers, in double and in a fixed order (one workgroup per sample).
 
-constexpr int kFinThreads = 1024;
 constexpr int kFinUnroll = 4;  // pairs a thread requests before it uses any
+// workgroup size: as few waves as request every pair in one round (fewer waves start sooner and
+// leave a shorter last loop), up to the largest workgroup
+inline int finalize_threads(int parts) {
+    const int t = (parts + kFinUnroll - 1) / kFinUnroll;
+    return t <= 256 ? 256 : t <= 512 ? 512 : 1024;
+}
 
 // (mean_i, M2_i) over `count` cells each -> (mean, rstd): mean = avg(mean_i),
 // M2 = sum(M2_i + count (mean_i - mean)^2)  (exact pairwise-combination formula).
-__global__ __launch_bounds__(kFinThreads) void ln_finalize_stats(const float *__restrict__ part,
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void ln_finalize_stats(const float *__restrict__ part,
                                                                  int parts, int count,
                                                                  float *__restrict__ stats, double eps) {
-    __shared__ double red[kFinThreads / kWave][3];
+    __shared__ double red[THREADS / kWave][3];
     const int tid = threadIdx.x, b = blockIdx.x;
     const float2 *ps = reinterpret_cast<const float2 *>(part) + (long)b * parts;
     double s = 0.0, q = 0.0, qm = 0.0;
     // one pass: sum(mean_i), sum(M2_i), sum(mean_i^2); means are O(1) and few thousand, so the
     // squares lose nothing in double
-    for (int i0 = tid; i0 < parts; i0 += kFinThreads * kFinUnroll) {
+    for (int i0 = tid; i0 < parts; i0 += THREADS * kFinUnroll) {
         float2 v[kFinUnroll];
 #pragma unroll
         for (int k = 0; k < kFinUnroll; ++k) {
-            const int i = i0 + k * kFinThreads;
+            const int i = i0 + k * THREADS;
             v[k] = i < parts ? ps[i] : make_float2(0.f, 0.f);
         }
 #pragma unroll
@@ -317,7 +323,7 @@ __global__ __launch_bounds__(kFinThreads) void ln_finalize_stats(const float *__
     __syncthreads();
     if (tid == 0) {
         s = q = qm = 0.0;
-        for (int w = 0; w < kFinThreads / kWave; ++w) {
+        for (int w = 0; w < THREADS / kWave; ++w) {
             s += red[w][0];
             q += red[w][1];
             qm += red[w][2];
@@ -331,18 +337,19 @@ __global__ __launch_bounds__(kFinThreads) void ln_finalize_stats(const float *__
 }
 
 // (s1_i, s2_i) -> (sum s1 / n, sum s2 / n)
-__global__ __launch_bounds__(kFinThreads) void ln_finalize_sums(const float *__restrict__ part,
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void ln_finalize_sums(const float *__restrict__ part,
                                                                 int parts, long n,
                                                                 float *__restrict__ sums) {
-    __shared__ double red[kFinThreads / kWave][2];
+    __shared__ double red[THREADS / kWave][2];
     const int tid = threadIdx.x, b = blockIdx.x;
     const float2 *ps = reinterpret_cast<const float2 *>(part) + (long)b * parts;
     double s1 = 0.0, s2 = 0.0;
-    for (int i0 = tid; i0 < parts; i0 += kFinThreads * kFinUnroll) {
+    for (int i0 = tid; i0 < parts; i0 += THREADS * kFinUnroll) {
         float2 v[kFinUnroll];
 #pragma unroll
         for (int k = 0; k < kFinUnroll; ++k) {
-            const int i = i0 + k * kFinThreads;
+            const int i = i0 + k * THREADS;
             v[k] = i < parts ? ps[i] : make_float2(0.f, 0.f);
         }
 #pragma unroll
@@ -360,7 +367,7 @@ __global__ __launch_bounds__(kFinThreads) void ln_finalize_sums(const float *__r
     __syncthreads();
     if (tid == 0) {
         s1 = s2 = 0.0;
-        for (int w = 0; w < kFinThreads / kWave; ++w) {
+        for (int w = 0; w < THREADS / kWave; ++w) {
             s1 += red[w][0];
             s2 += red[w][1];
         }
@@ -448,15 +455,34 @@ template <typename T> int backward_t(const LayerNormArgs &a, hipStream_t st) {
 
 int layernorm_finalize_stats(const float *part, int parts_per_sample, int count, float *stats, int B,
                              double eps, hipStream_t st) {
-    hipLaunchKernelGGL(ln_finalize_stats, dim3(B), dim3(kFinThreads), 0, st, part, parts_per_sample,
-                       count, stats, eps);
+    switch (finalize_threads(parts_per_sample)) {
+    case 256:
+        hipLaunchKernelGGL(ln_finalize_stats<256>, dim3(B), dim3(256), 0, st, part, parts_per_sample, count,
+                           stats, eps);
+        break;
+    case 512:
+        hipLaunchKernelGGL(ln_finalize_stats<512>, dim3(B), dim3(512), 0, st, part, parts_per_sample, count,
+                           stats, eps);
+        break;
+    default:
+        hipLaunchKernelGGL(ln_finalize_stats<1024>, dim3(B), dim3(1024), 0, st, part, parts_per_sample, count,
+                           stats, eps);
+    }
     return check_launch("ln_finalize_stats");
 }
 
 int layernorm_finalize_sums(const float *part, int parts_per_sample, long n, float *sums, int B,
                             hipStream_t st) {
-    hipLaunchKernelGGL(ln_finalize_sums, dim3(B), dim3(kFinThreads), 0, st, part, parts_per_sample, n,
-                       sums);
+    switch (finalize_threads(parts_per_sample)) {
+    case 256:
+        hipLaunchKernelGGL(ln_finalize_sums<256>, dim3(B), dim3(256), 0, st, part, parts_per_sample, n, sums);
+        break;
+    case 512:
+        hipLaunchKernelGGL(ln_finalize_sums<512>, dim3(B), dim3(512), 0, st, part, parts_per_sample, n, sums);
+        break;
+    default:
+        hipLaunchKernelGGL(ln_finalize_sums<1024>, dim3(B), dim3(1024), 0, st, part, parts_per_sample, n, sums);
+    }
     return check_launch("ln_finalize_sums");
 }
 
