@@ -442,8 +442,12 @@ void step_fwd_split(
     // committed (see step_fwd_fast).
     float done[4];
     int done_s = -1;
+    // Turns pay when the grid is a single round of workgroups (the batch was split to fill the
+    // chip: nchunk > 1).  With one workgroup per block and more blocks than the chip holds, a
+    // workgroup that ends early is replaced at once, and the turns cost 1.5 % (128^3, batch 8).
+    const bool turns = nchunk > 1;
     for (int s = s0; s < s1; ++s) {
-        take_turns(s);
+        if (turns) take_turns(s);
         commit(lds, 2, pre, ln_in, pre_mean, pre_rstd);
         if (NORM) {
             shift = pre_shift;
