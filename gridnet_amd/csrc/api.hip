@@ -2,6 +2,7 @@
 // Nothing here allocates, frees or synchronises; every entry point only enqueues kernels.
 
 #include <cstring>
+#include <mutex>
 
 #include "common.h"
 #include "launch.h"
@@ -60,11 +61,46 @@ int check_step(const StepArgs &a, bool backward, bool gated = false) {
 }  // namespace
 }  // namespace gridnet
 
+// ---- scratch for the entry point that takes no workspace ----------------------------------
+// One array per GPU (every device that loads this code object gets its own copy at its own
+// address), held until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress, not a device address: kernels are given the looked-up pointer.
+static __device__ __align__(256) unsigned char scratch[GRIDNET_STATIC_SCRATCH_BYTES];
+
+namespace gridnet {
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex scratch_lock;
+void *scratch_ptr[kMaxDevices];  // by device ordinal, looked up on first use with that device current
+
+int static_scratch_pointer(void **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return fail(GRIDNET_ERR_LAUNCH, "static scratch: no usable current device (%s, ordinal %d)",
+                    hipGetErrorString(e), dev);
+    std::lock_guard<std::mutex> hold(scratch_lock);
+    if (!scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return fail(GRIDNET_ERR_LAUNCH, "static scratch: hipGetSymbolAddress failed on device %d: %s",
+                        dev, hipGetErrorString(e));
+        scratch_ptr[dev] = p;
+    }
+    *out = scratch_ptr[dev];
+    return GRIDNET_OK;
+}
+
+}  // namespace
+}  // namespace gridnet
+
 using namespace gridnet;
 
 extern "C" {
 
-int gridnet_hip_version(void) { return 4; }  // 2: fused body; 3: residual forward and backward; 4: gated backward takes a workspace
+int gridnet_hip_version(void) { return 5; }  // 2: fused body; 3: residual forward and backward; 4: gated backward takes a workspace; 5: backward on static scratch
 
 const char *gridnet_hip_last_error(void) { return error_buffer(); }
 
@@ -103,28 +139,61 @@ size_t gridnet_hip_backward_workspace_bytes(int dtype, int B, int M, int N, int 
     return 0;
 }
 
-int gridnet_hip_backward(int dtype, const void *weight, const void *bias, const void *scale,
+static int backward_step(int dtype, const void *weight, const void *bias, const void *scale,
                          const void *x, const void *dy, void *dweight, void *dbias, void *dscale,
                          void *dx, int B, int M, int N, int K, int inner, int block_size,
                          double eps, int normalize, int activation, int flags, void *workspace,
-                         size_t workspace_bytes, void *stream) {
+                         size_t workspace_bytes, void *stream, bool static_scratch) {
     StepArgs a{};
     a.dtype = dtype; a.weight = weight; a.bias = bias; a.scale = scale; a.x = x; a.dy = dy;
     a.dweight = dweight; a.dbias = dbias; a.dscale = dscale; a.dx = dx;
     a.B = B; a.M = M; a.N = N; a.K = K; a.inner = inner; a.block_size = block_size;
     a.eps = eps; a.normalize = normalize != 0; a.activation = activation; a.flags = flags;
-    a.workspace = workspace; a.workspace_bytes = workspace_bytes;
     if (int rc = check_step(a, true)) return rc;
     if (B == 0) return GRIDNET_OK;
     hipStream_t st = (hipStream_t)stream;
-    if (step_fast_supports(a, true)) {
-        const size_t need = step_fast_backward_workspace(a);
-        if (need && (!workspace || workspace_bytes < need))
-            return fail(GRIDNET_ERR_WORKSPACE, "backward needs %zu bytes of workspace, got %zu", need,
-                        workspace ? workspace_bytes : (size_t)0);
-        return step_backward_fast(a, st);
+    if (!step_fast_supports(a, true)) return step_backward_generic(a, st);  // needs no scratch
+    const size_t need = step_fast_backward_workspace(a);
+    if (static_scratch) {
+        // sizes first: a problem that does not fit is refused before anything touches the device
+        if (need > (size_t)GRIDNET_STATIC_SCRATCH_BYTES)
+            return fail(GRIDNET_ERR_WORKSPACE,
+                        "backward needs %zu bytes of scratch, the static array holds %zu: use "
+                        "gridnet_hip_backward with a workspace",
+                        need, (size_t)GRIDNET_STATIC_SCRATCH_BYTES);
+        if (int rc = static_scratch_pointer(&workspace)) return rc;
+        workspace_bytes = GRIDNET_STATIC_SCRATCH_BYTES;
     }
-    return step_backward_generic(a, st);
+    if (need && (!workspace || workspace_bytes < need))
+        return fail(GRIDNET_ERR_WORKSPACE, "backward needs %zu bytes of workspace, got %zu", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    a.workspace = workspace; a.workspace_bytes = workspace_bytes;
+    return step_backward_fast(a, st);
+}
+
+int gridnet_hip_backward(int dtype, const void *weight, const void *bias, const void *scale,
+                         const void *x, const void *dy, void *dweight, void *dbias, void *dscale,
+                         void *dx, int B, int M, int N, int K, int inner, int block_size,
+                         double eps, int normalize, int activation, int flags, void *workspace,
+                         size_t workspace_bytes, void *stream) {
+    return backward_step(dtype, weight, bias, scale, x, dy, dweight, dbias, dscale, dx, B, M, N, K,
+                         inner, block_size, eps, normalize, activation, flags, workspace,
+                         workspace_bytes, stream, false);
+}
+
+int gridnet_hip_static_init(void) {
+    void *unused = nullptr;
+    return static_scratch_pointer(&unused);
+}
+
+int gridnet_hip_backward_static(int dtype, const void *weight, const void *bias, const void *scale,
+                                const void *x, const void *dy, void *dweight, void *dbias,
+                                void *dscale, void *dx, int B, int M, int N, int K, int inner,
+                                int block_size, double eps, int normalize, int activation,
+                                int flags, void *stream) {
+    return backward_step(dtype, weight, bias, scale, x, dy, dweight, dbias, dscale, dx, B, M, N, K,
+                         inner, block_size, eps, normalize, activation, flags, nullptr, 0, stream,
+                         true);
 }
 
 int gridnet_hip_forward_gated(int dtype, const void *weight, const void *bias, const void *x, void *y,

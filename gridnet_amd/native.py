@@ -19,6 +19,7 @@ F32, F64 = 0, 1
 OVERWRITE_PARAMS = 1
 OVERWRITE_DX = 2
 OVERWRITE = 3
+STATIC_SCRATCH_BYTES = 40 << 20  # GRIDNET_STATIC_SCRATCH_BYTES
 
 EXPORTS = (
     "gridnet_hip_version",
@@ -27,6 +28,8 @@ EXPORTS = (
     "gridnet_hip_forward",
     "gridnet_hip_backward_workspace_bytes",
     "gridnet_hip_backward",
+    "gridnet_hip_static_init",
+    "gridnet_hip_backward_static",
     "gridnet_hip_forward_gated",
     "gridnet_hip_backward_gated_workspace_bytes",
     "gridnet_hip_backward_gated",
@@ -67,6 +70,10 @@ def _load():
     lib.gridnet_hip_backward.restype = i
     lib.gridnet_hip_backward.argtypes = [i, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, d, i, i, i,
                                          p, z, p]
+    lib.gridnet_hip_static_init.restype = i
+    lib.gridnet_hip_static_init.argtypes = []
+    lib.gridnet_hip_backward_static.restype = i
+    lib.gridnet_hip_backward_static.argtypes = [i, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, d, i, i, i, p]
     lib.gridnet_hip_forward_gated.restype = i
     lib.gridnet_hip_forward_gated.argtypes = [i, p, p, p, p, i, i, i, i, i, i, i, p]
     lib.gridnet_hip_backward_gated_workspace_bytes.restype = z

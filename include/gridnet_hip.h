@@ -104,6 +104,32 @@ int gridnet_hip_backward(int dtype, const void *weight, const void *bias, const 
                          void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * gridnet_hip_backward without a workspace argument and without any allocation.  It has no
+ * counterpart in the reference; it exists for callers that cannot allocate device memory:
+ * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
+ * The scratch that gridnet_hip_backward takes as `workspace` lives in a static device array of
+ * GRIDNET_STATIC_SCRATCH_BYTES inside the library instead (one copy per GPU, held until the
+ * process ends).  A problem that needs more (gridnet_hip_backward_workspace_bytes() tells) is
+ * rejected with GRIDNET_ERR_WORKSPACE and nothing is enqueued.  Same arguments, results and
+ * flags as gridnet_hip_backward otherwise (it runs the same kernels).
+ * Every call on a GPU shares that GPU's array: calls that may overlap on one GPU (different
+ * streams, different threads) race and must be serialised by the caller.  The array's
+ * contents need not be, and are not, preserved between calls.
+ * gridnet_hip_static_init() looks the array up for the CURRENT device (hipGetSymbolAddress; no
+ * allocation either); gridnet_hip_backward_static does the same on its first call on a
+ * device, so a caller that is going to capture a graph calls the init once beforehand.
+ */
+#define GRIDNET_STATIC_SCRATCH_BYTES (40u << 20)
+
+int gridnet_hip_static_init(void);
+
+int gridnet_hip_backward_static(int dtype, const void *weight, const void *bias, const void *scale,
+                                const void *x, const void *dy, void *dweight, void *dbias,
+                                void *dscale, void *dx, int B, int M, int N, int K, int inner,
+                                int block_size, double eps, int normalize, int activation,
+                                int flags, void *stream);
+
+/*
  * Gated variant: x' = gate*x + (1-gate)*act(pre), weight [27,2,M,N,K] (channel 0: pre,
  * channel 1: gate), bias [2,M,N,K]; no scale, eps or normalisation.  Replace
  * gated_gridnet_cuda_forward / gated_gridnet_cuda_backward, src/gridnet_cuda_kernels.cu:853-930

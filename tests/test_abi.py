@@ -72,6 +72,11 @@ def test_host_only_entry_points():
     rc = native.lib.gridnet_hip_backward(0, 8, 8, 8, 8, 8, 8, 8, 8, 8, 2, 8, 8, 8, 2, 8, 1e-5, 1, 0, 0,
                                          None, 0, None)
     assert rc == 4 and "workspace" in native.last_error()
+    # the entry point on static scratch refuses, before touching a device, what its array cannot hold
+    assert native.lib.gridnet_hip_backward_workspace_bytes(0, 64, 64, 64, 64, 4, 8, 0) > native.STATIC_SCRATCH_BYTES
+    rc = native.lib.gridnet_hip_backward_static(0, 8, 8, 8, 8, 8, 8, 8, 8, 8, 64, 64, 64, 64, 4, 8, 1e-5,
+                                                0, 0, 0, None)
+    assert rc == 4 and "static array holds" in native.last_error()
     assert native.lib.gridnet_hip_layernorm_workspace_bytes(0, 32, 64 ** 3) == (32 * 64 * 2 + 64) * 4
     rc = native.lib.gridnet_hip_layernorm_forward(0, 8, 8, 8, 8, 8, 8, 4, 4096, 1e-5, None, 0, None)
     assert rc == 4 and "workspace" in native.last_error()
