@@ -146,6 +146,67 @@ def cpu_baseline(wl, budget_s=25.0):
     }
 
 
+def reference_benchmark_shape(steps, warmup):
+    """The reference's own benchmark (gridnet/backend_cuda_test.py:155-206; it stores no result):
+    32^3 grid, batch 2, 10 inner iterations, 8^3 blocks, normalize=True, silu, all parameters
+    N(0, 1), ONE op call through the autograd wrapper with a synchronisation after every call, as
+    its harness does -- forward alone, forward + backward, and the gated twin (leaky_relu)."""
+    import torch
+
+    from gridnet_amd.backend_cuda import GatedGridnetCudaOp, GridnetCudaOp
+
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    shape = (32, 32, 32)
+    x = torch.randn(2, *shape, device=dev, requires_grad=True)
+    w = torch.randn(27, *shape, device=dev, requires_grad=True)
+    b = torch.randn(*shape, device=dev, requires_grad=True)
+    r = torch.randn(*shape, device=dev, requires_grad=True)
+    wg = torch.randn(27, 2, *shape, device=dev, requires_grad=True)
+    bg = torch.randn(2, *shape, device=dev, requires_grad=True)
+    gy = torch.randn_like(x)
+
+    def fwd():
+        with torch.no_grad():
+            GridnetCudaOp.apply(w, b, r, x, 10, 8, 1e-5, True, "silu")
+        torch.cuda.synchronize()
+
+    def fwd_bwd():
+        out = GridnetCudaOp.apply(w, b, r, x, 10, 8, 1e-5, True, "silu")
+        torch.autograd.grad(out, (x, w, b, r), gy)
+        torch.cuda.synchronize()
+
+    def gated_fwd_bwd():
+        out = GatedGridnetCudaOp.apply(wg, bg, x, 10, 8, "leaky_relu")
+        torch.autograd.grad(out, (x, wg, bg), gy)
+        torch.cuda.synchronize()
+
+    def clock(fn):
+        for _ in range(warmup):
+            fn()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        return (time.perf_counter() - t0) / steps
+
+    t_f, t_fb, t_g = clock(fwd), clock(fwd_bwd), clock(gated_fwd_bwd)
+    cu = 2 * 32 ** 3 * 10
+    a, p = 2 * 32 ** 3 * 4, 32 ** 3 * 4
+    algo = (2 * a + 29 * p) + (3 * a + 58 * p)  # one step forward, one step backward
+    print(json.dumps({
+        "metric": "cell-updates/s fwd+bwd, 64^3 grid 8^3 blocks batch 32; % of HBM roofline",
+        "value": cu / t_fb, "unit": "cell-updates/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": t_fb * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "R 32^3 bs8 B2 inner10 normalize silu: the reference's own benchmark "
+                               "shape and harness (one op call, synchronised, through autograd)",
+                   "pass": "fwd+bwd"},
+        "forward_only_ms": t_f * 1e3, "gated_fwd_bwd_ms": t_g * 1e3,
+        "hbm_roofline_frac_whole_step": algo / t_fb / (HBM_PEAK_GBS * 1e9),
+        "note": "a 64-block grid and two samples: host- and latency-bound, not a throughput shape",
+    }), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -168,6 +229,8 @@ def main():
                  "use --gpus 1")
     from gridnet_amd.configs import WORKLOADS
 
+    if args.workload == "R":
+        return reference_benchmark_shape(args.steps, args.warmup)
     wl = WORKLOADS[args.workload]
     if args.normalize:
         wl = dataclasses.replace(wl, normalize=True, name=wl.name + " normalize")

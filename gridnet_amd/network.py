@@ -33,12 +33,21 @@ class FusedBodyOp(torch.autograd.Function):
                          activation, backward=need_grad, fused=True, outer_residual=outer_residual)
         y = run.forward(x0.detach().contiguous())
         ctx.run = run if need_grad else None
+        if need_grad:
+            # the runner reads these tensors again in the backward (it recomputes from them):
+            # registering them lets autograd refuse a backward after an in-place change, such as
+            # an optimizer step taken while this forward was still outstanding
+            ctx.save_for_backward(x0, weight, bias, scale, gamma, beta)
         return y
 
     @staticmethod
     @once_differentiable
     def backward(ctx, grad_out):
         run, ctx.run = ctx.run, None
+        if run is None:
+            raise RuntimeError("FusedBodyOp: the buffers of this forward were released by its first "
+                               "backward; a second backward (retain_graph=True) is not supported")
+        ctx.saved_tensors  # raises if an input was modified in place since the forward
         dw, db, dr, dgamma, dbeta, dx0 = run.backward(grad_out.contiguous())
         return dx0, dw, db, dr, dgamma, dbeta, None, None, None, None, None
 

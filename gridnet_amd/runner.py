@@ -27,6 +27,8 @@ class BodyRunner:
                  fused: bool = False, outer_residual: bool = False):
         self.w, self.b, self.r, self.gamma, self.beta = weight, bias, scale, gamma, beta
         self.B, (self.M, self.N, self.K) = batch, bias.shape
+        if outer < 1:
+            raise ValueError(f"outer must be at least 1, got {outer}")
         self.inner, self.outer, self.bs = inner, outer, block_size
         self.act = _n.activation_id(activation)
         self.normalize, self.eps, self.ln_eps = int(normalize), eps, ln_eps
@@ -36,9 +38,19 @@ class BodyRunner:
         self.n = n
         shape = (batch, self.M, self.N, self.K)
         keep = outer if backward else 1
-        # h[j]: input of outer step j (h[outer] = result); s[j]: its output before the norm
-        self.h = [torch.empty(shape, device=dev, dtype=dtype) for _ in range(keep + 1)]
-        self.s = [torch.empty(shape, device=dev, dtype=dtype) for _ in range(keep)]
+        if outer_residual and not fused:
+            raise RuntimeError("outer_residual runs through the fused entry points only (fused=True)")
+        # h[j]: input of outer step j (h[outer] = result); s[j]: its output before the norm.
+        # What a mode never touches is not allocated: the fused chain keeps the raw outputs s[*]
+        # and one h (the final result; forward only, a second buffer to alternate with), the
+        # residual chain every h and two s (free buffers for its backward).
+        n_h, n_s = keep + 1, keep
+        if fused and not outer_residual:
+            n_h = 1 if backward else 2
+        if fused and outer_residual:
+            n_s = 2 if backward else 1
+        self.h = [torch.empty(shape, device=dev, dtype=dtype) for _ in range(n_h)]
+        self.s = [torch.empty(shape, device=dev, dtype=dtype) for _ in range(n_s)]
         self.mean = torch.empty(keep, batch, device=dev, dtype=dtype)
         self.rstd = torch.empty(keep, batch, device=dev, dtype=dtype)
         self.ln_ws_bytes = _n.lib.gridnet_hip_layernorm_workspace_bytes(self.dt, batch, n)
@@ -58,8 +70,6 @@ class BodyRunner:
         self.on_launch = None  # optional hook(name, phase) for per-kernel timing
         self.fused = fused
         self.outer_residual = outer_residual
-        if outer_residual and not fused:
-            raise RuntimeError("outer_residual runs through the fused entry points only (fused=True)")
         if fused:
             if weight.dtype != torch.float32 or normalize or inner < 1:
                 raise RuntimeError("the fused body covers float32, normalize=False, inner >= 1")

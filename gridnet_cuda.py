@@ -14,12 +14,34 @@ from gridnet_amd import native as _n
 __all__ = ["forward", "backward", "forward_gated", "backward_gated"]
 
 
+def _check_call(named, activations):
+    """Host-side checks that the native side relies on.  The reference's binding gets them from
+    its typed, sized accessors (``packed_accessor32<scalar_t, N>`` raises on a dtype or rank
+    mismatch and bounds every index, src/gridnet_cuda.cpp:103-107); raw pointers do not, and an
+    out-of-bounds access on the device is a fault, not an exception.  ``named``: (tensor, name,
+    expected shape) triples; every tensor must be a contiguous HIP tensor of the first one's
+    dtype and device."""
+    ref = named[0][0]
+    for t, name, _ in named:
+        _n.check_input(t, name)
+    if activations.dim() != 4:
+        raise RuntimeError(f"initActivations must be [B, M, N, K], got {tuple(activations.shape)}")
+    for t, name, shape in named:
+        if t.dtype != ref.dtype:
+            raise RuntimeError(f"{name} has dtype {t.dtype}, expected {ref.dtype} like {named[0][1]}")
+        if t.device != ref.device:
+            raise RuntimeError(f"{name} is on {t.device}, expected {ref.device} like {named[0][1]}")
+        if tuple(t.shape) != tuple(shape):
+            raise RuntimeError(f"{name} has shape {tuple(t.shape)}, expected {tuple(shape)}")
+
+
 def forward(weight, bias, scale, initActivations, outActivations, innerIterations, blockSize,
             eps, normalize, activation):
     """One outer step; replaces gridnet_forward, src/gridnet_cuda.cpp:61-89."""
-    for t, name in ((weight, "weight"), (bias, "bias"), (scale, "scale"),
-                    (initActivations, "initActivations"), (outActivations, "outActivations")):
-        _n.check_input(t, name)
+    grid, x = tuple(initActivations.shape[1:]), tuple(initActivations.shape)
+    _check_call(((weight, "weight", (27, *grid)), (bias, "bias", grid), (scale, "scale", grid),
+                 (initActivations, "initActivations", x), (outActivations, "outActivations", x)),
+                initActivations)
     act = _n.activation_id(activation)
     B, M, N, K = initActivations.shape
     with torch.cuda.device(weight.device):
@@ -38,11 +60,12 @@ def backward(weight, bias, scale, initActivations, outGrads, weightGradOut, bias
     As in the reference the four gradient outputs are accumulated into (its wrapper hands
     them over zero-filled, gridnet/backend_cuda.py:78-81).
     """
-    for t, name in ((weight, "weight"), (bias, "bias"), (scale, "scale"),
-                    (initActivations, "initActivations"), (outGrads, "outGrads"),
-                    (weightGradOut, "weightGradOut"), (biasGradOut, "biasGradOut"),
-                    (scaleGradOut, "scaleGradOut"), (activationsGradOut, "activationsGradOut")):
-        _n.check_input(t, name)
+    grid, x = tuple(initActivations.shape[1:]), tuple(initActivations.shape)
+    _check_call(((weight, "weight", (27, *grid)), (bias, "bias", grid), (scale, "scale", grid),
+                 (initActivations, "initActivations", x), (outGrads, "outGrads", x),
+                 (weightGradOut, "weightGradOut", (27, *grid)), (biasGradOut, "biasGradOut", grid),
+                 (scaleGradOut, "scaleGradOut", grid), (activationsGradOut, "activationsGradOut", x)),
+                initActivations)
     act = _n.activation_id(activation)
     B, M, N, K = initActivations.shape
     dt = _n.dtype_id(weight)
@@ -61,9 +84,10 @@ def backward(weight, bias, scale, initActivations, outGrads, weightGradOut, bias
 def forward_gated(weight, bias, initActivations, outActivations, innerIterations, blockSize,
                   activation):
     """Gated outer step; replaces gated_gridnet_forward, src/gridnet_cuda.cpp:133-158."""
-    for t, name in ((weight, "weight"), (bias, "bias"), (initActivations, "initActivations"),
-                    (outActivations, "outActivations")):
-        _n.check_input(t, name)
+    grid, x = tuple(initActivations.shape[1:]), tuple(initActivations.shape)
+    _check_call(((weight, "weight", (27, 2, *grid)), (bias, "bias", (2, *grid)),
+                 (initActivations, "initActivations", x), (outActivations, "outActivations", x)),
+                initActivations)
     act = _n.activation_id(activation)
     B, M, N, K = initActivations.shape
     with torch.cuda.device(weight.device):
@@ -77,10 +101,13 @@ def backward_gated(weight, bias, initActivations, outGrads, weightGradOut, biasG
                    activationsGradOut, innerIterations, blockSize, activation):
     """Backward of the gated step; replaces gated_gridnet_backward, src/gridnet_cuda.cpp:160-186.
     Gradient outputs are accumulated into, as in the reference."""
-    for t, name in ((weight, "weight"), (bias, "bias"), (initActivations, "initActivations"),
-                    (outGrads, "outGrads"), (weightGradOut, "weightGradOut"),
-                    (biasGradOut, "biasGradOut"), (activationsGradOut, "activationsGradOut")):
-        _n.check_input(t, name)
+    grid, x = tuple(initActivations.shape[1:]), tuple(initActivations.shape)
+    _check_call(((weight, "weight", (27, 2, *grid)), (bias, "bias", (2, *grid)),
+                 (initActivations, "initActivations", x), (outGrads, "outGrads", x),
+                 (weightGradOut, "weightGradOut", (27, 2, *grid)),
+                 (biasGradOut, "biasGradOut", (2, *grid)),
+                 (activationsGradOut, "activationsGradOut", x)),
+                initActivations)
     act = _n.activation_id(activation)
     B, M, N, K = initActivations.shape
     dt = _n.dtype_id(weight)

@@ -109,6 +109,56 @@ def test_shim_rejects_host_tensors_like_the_reference_binding():
         gridnet_cuda.forward(w, p, p, t, t.clone(), 1, 8, 1e-5, False, "silu")
 
 
+def test_shim_validates_dtypes_and_shapes_on_the_host(monkeypatch):
+    """Raw pointers carry no dtype or size: what the reference's typed accessors would refuse
+    (src/gridnet_cuda.cpp:103-107) is refused here before any native call.  The device check is
+    patched out so that host tensors reach the checks behind it."""
+    import torch
+
+    import gridnet_cuda
+    from gridnet_amd import native
+
+    monkeypatch.setattr(native, "check_input", lambda t, name: None)
+
+    def forbid(*a, **k):
+        raise AssertionError("a native entry point was reached")
+
+    for name in ("gridnet_hip_forward", "gridnet_hip_backward", "gridnet_hip_forward_gated",
+                 "gridnet_hip_backward_gated"):
+        monkeypatch.setattr(native.lib, name, forbid)
+    w, p, x = torch.zeros(27, 8, 8, 16), torch.zeros(8, 8, 16), torch.zeros(2, 8, 8, 16)
+    ok = (w, p, p, x, x.clone())
+    cases = {
+        "bias has dtype": (w, p.double(), p, x, x.clone()),
+        "initActivations has dtype": (w, p, p, x.double(), x.clone()),
+        "outActivations has shape": (w, p, p, x, x[:1].clone()),
+        "weight has shape": (w[:, :, :, :8].contiguous(), p, p, x, x.clone()),
+        "scale has shape": (w, p, p[:4].contiguous(), x, x.clone()),
+    }
+    for message, args in cases.items():
+        with pytest.raises(RuntimeError, match=message):
+            gridnet_cuda.forward(*args, 1, 8, 1e-5, False, "silu")
+    grads = (torch.zeros_like(w), torch.zeros_like(p), torch.zeros_like(p), torch.zeros_like(x))
+    with pytest.raises(RuntimeError, match="weightGradOut has shape"):
+        gridnet_cuda.backward(w, p, p, x, x.clone(), grads[0][:26].contiguous(), *grads[1:], 1, 8, 1e-5,
+                              False, "silu")
+    with pytest.raises(RuntimeError, match="activationsGradOut has dtype"):
+        gridnet_cuda.backward(w, p, p, x, x.clone(), *grads[:3], grads[3].double(), 1, 8, 1e-5, False,
+                              "silu")
+    with pytest.raises(RuntimeError, match="outGrads has shape"):
+        gridnet_cuda.backward(w, p, p, x, x[:1].clone(), *grads, 1, 8, 1e-5, False, "silu")
+    wg, pg = torch.zeros(27, 2, 8, 8, 16), torch.zeros(2, 8, 8, 16)
+    with pytest.raises(RuntimeError, match="weight has shape"):
+        gridnet_cuda.forward_gated(w, pg, x, x.clone(), 1, 8, "tanh")
+    with pytest.raises(RuntimeError, match="biasGradOut has shape"):
+        gridnet_cuda.backward_gated(wg, pg, x, x.clone(), torch.zeros_like(wg), torch.zeros_like(p),
+                                    torch.zeros_like(x), 1, 8, "tanh")
+    with pytest.raises(RuntimeError, match=r"must be \[B, M, N, K\]"):
+        gridnet_cuda.forward(w, p, p, x[0], x[0].clone(), 1, 8, 1e-5, False, "silu")
+    # and a well-formed call passes every check
+    gridnet_cuda._check_call(tuple(zip(ok, "abcde", [(27, 8, 8, 16), (8, 8, 16), (8, 8, 16), x.shape, x.shape])), x)
+
+
 def test_dispatcher_never_falls_back():
     import torch
 

@@ -62,6 +62,54 @@ def test_random_step_tuned_fp32_against_generic_fp64(seed):
                      what=name)
 
 
+def draw_kinked(seed):
+    """Draws under relu / leaky_relu, sized so that inputs exist which keep every pre-activation
+    of the fp64 run clear of the kink (cells x batch x iterations below ~2e5)."""
+    rng = random.Random(9000 + seed)
+    bs = rng.choice((4, 8))
+    dims = tuple(bs * rng.randint(1, 3) for _ in range(3))
+    inner = rng.choice((1, 1, 2, 3, 4, 5))
+    cells = dims[0] * dims[1] * dims[2]
+    fits = [b for b in (1, 2, 3, 5, 7, 9, 13, 17, 31, 33) if b * cells * inner <= 200_000]
+    return dims, bs, rng.choice(fits[-4:]), inner, rng.choice(("relu", "leaky_relu")), rng.random() < 0.5
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_step_kinked_activations(seed):
+    """relu and leaky_relu (the training default) through the same launch plans: batches that
+    the slots do not divide, batches split over workgroups, preset gradient buffers.  The
+    derivative jumps at 0, so the inputs are chosen with every fp64 pre-activation at least
+    2e-6 away from it (ten times what fp32 rounding moves one by)."""
+    import gridnet_cuda
+    from helpers import acts_clear_of_kink
+
+    shape, bs, batch, inner, activation, preset = draw_kinked(seed)
+    print(f"sweep kinked seed={seed} shape={shape} bs={bs} B={batch} inner={inner} act={activation} "
+          f"preset={preset}", flush=True)
+    w, b, r = make_params(shape, seed=9100 + seed)
+    if inner >= 5:
+        w, r = w * 0.5, r * 0.5
+    x = acts_clear_of_kink(w, b, r, batch, shape, inner, bs, 1e-5, False, activation, seed=9200 + seed)
+    gy = make_acts(batch, shape, seed=9300 + seed)
+    start = [make_acts(1, t.shape, seed=9400 + seed + i)[0] if preset else torch.zeros_like(t)
+             for i, t in enumerate((w, b, r, x))]
+
+    def call(dtype):
+        tw, tb, tr, tx, tgy = (t.to(device=DEV, dtype=dtype) for t in (w, b, r, x, gy))
+        y = torch.full_like(tx, float("nan"))
+        gridnet_cuda.forward(tw, tb, tr, tx, y, inner, bs, 1e-5, False, activation)
+        outs = [t.to(device=DEV, dtype=dtype) for t in start]
+        gridnet_cuda.backward(tw, tb, tr, tx, tgy, *outs, inner, bs, 1e-5, False, activation)
+        return [y] + outs
+
+    fast, slow = call(torch.float32), call(torch.float64)
+    summed = 1e-5 * max(1.0, math.sqrt(batch * inner / 2))
+    for name, got, want in zip(("y", "dweight", "dbias", "dscale", "dx"), fast, slow):
+        assert torch.isfinite(got).all(), name
+        assert_close(got, want, atol=summed if name in ("dweight", "dbias", "dscale") else 1e-5,
+                     what=name)
+
+
 def draw_normalized(seed):
     if seed == 0:  # the draw that once showed a missing barrier in the tuned backward
         return (24, 24, 24), 8, 40, 1, "tanh"
