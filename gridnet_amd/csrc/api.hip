@@ -491,4 +491,71 @@ int gridnet_hip_fused_backward_residual(int dtype, const void *weight, const voi
                           g_out);
 }
 
+int gridnet_hip_chain_supported(int dtype, int inner, int block_size, int normalize) {
+    StepArgs a{};
+    a.dtype = dtype; a.inner = inner; a.block_size = block_size; a.normalize = normalize != 0;
+    return chain_supports(a) ? 1 : 0;
+}
+
+size_t gridnet_hip_chain_halo_floats(int B, int M, int N, int K, int block_size) {
+    if (B <= 0 || M <= 0 || N <= 0 || K <= 0 || block_size != 8) return 0;
+    StepArgs a{};
+    a.B = B; a.M = M; a.N = N; a.K = K; a.block_size = block_size;
+    return chain_halo_floats(a);
+}
+
+int gridnet_hip_chain_backward(int dtype, const void *weight, const void *bias, const void *scale,
+                               const void *gamma, const void *beta, const void *x,
+                               const void *x_stats, const void *dy, const void *y_raw,
+                               const void *y_stats, const void *y_sums, const void *halo_in,
+                               void *halo_out, void *dweight, void *dbias, void *dscale, void *dgamma,
+                               void *dbeta, void *dx, void *x_sums, int B, int M, int N, int K,
+                               int inner, int block_size, int activation, int flags, void *workspace,
+                               size_t workspace_bytes, void *stream) {
+    StepArgs a{};
+    a.dtype = dtype; a.weight = weight; a.bias = bias; a.scale = scale;
+    a.x = x; a.dy = dy; a.dweight = dweight; a.dbias = dbias; a.dscale = dscale; a.dx = dx;
+    a.B = B; a.M = M; a.N = N; a.K = K; a.inner = inner; a.block_size = block_size;
+    a.activation = activation;
+    a.flags = (flags & GRIDNET_OVERWRITE_PARAMS) | GRIDNET_OVERWRITE_DX;  // dx is always written
+    a.ln.gamma = (const float *)gamma;
+    if (!chain_supports(a))
+        return fail(GRIDNET_ERR_ARGUMENT,
+                    "the chain entry points cover float32, block_size 8 and 1 to 4 inner iterations "
+                    "(dtype id %d, block_size %d, inner %d): use gridnet_hip_fused_backward",
+                    dtype, block_size, inner);
+    if (int rc = check_fused(a, true)) return rc;
+    if (B == 0) return GRIDNET_OK;
+    if (!gamma || !beta || !dgamma || !dbeta || !y_raw || !y_stats || !y_sums)
+        return fail(GRIDNET_ERR_ARGUMENT, "null pointer");
+    if ((x_stats == nullptr) != (x_sums == nullptr))
+        return fail(GRIDNET_ERR_ARGUMENT, "x_stats and x_sums go together: both or neither");
+    if (halo_out && !x_stats)
+        return fail(GRIDNET_ERR_ARGUMENT,
+                    "an unfinished dx (halo_out) is for a step whose input passes a LayerNorm: "
+                    "x_stats and x_sums are required");
+    const size_t dsum_bytes = fused_backward_dsum(a), need = dsum_bytes + fused_backward_parts(a);
+    if (!workspace || workspace_bytes < need)
+        return fail(GRIDNET_ERR_WORKSPACE, "chain backward needs %zu bytes of workspace, got %zu", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    hipStream_t st = (hipStream_t)stream;
+    a.workspace = workspace; a.workspace_bytes = dsum_bytes;
+    a.ln.beta = (const float *)beta;
+    a.ln.x_stats = (const float *)x_stats;
+    a.ln.y_raw = (const float *)y_raw;
+    a.ln.y_stats = (const float *)y_stats;
+    a.ln.y_sums = (const float *)y_sums;
+    a.ln.dgamma = (float *)dgamma;
+    a.ln.dbeta = (float *)dbeta;
+    a.ln.x_part = x_stats ? (float *)((char *)workspace + dsum_bytes) : nullptr;
+    a.ln.halo_in = (const float *)halo_in;
+    a.ln.halo_out = (float *)halo_out;
+    a.ln.g_rows = (const float *)dy;
+    if (int rc = chain_backward(a, st)) return rc;
+    if (!x_stats) return GRIDNET_OK;
+    const int nblk = (M / block_size) * (N / block_size) * (K / block_size);
+    return layernorm_finalize_sums(a.ln.x_part, nblk * step_fast_backward_parts(block_size),
+                                   (long)M * N * K, (float *)x_sums, B, st);
+}
+
 }  // extern "C"

@@ -6,6 +6,7 @@
 #define GRIDNET_FAST_TILES_H
 
 #include "common.h"
+#include "launch.h"
 
 namespace gridnet {
 namespace {
@@ -241,14 +242,19 @@ template <typename TL, int NT = TL::TPS> struct Fetch {  // NT: threads of a slo
             goff[e] = (ok[e] ? (gi * N + gj) * K : 0) + r0 + half * HC;
         }
     }
-    // Unconditional loads (no branches, no register initialisation in front of them).
+    // Unconditional loads (no branches, no register initialisation in front of them).  The lane
+    // offsets are handed over as unsigned BYTE offsets beside the uniform base: that is an
+    // addressing mode (scalar base + 32-bit lane offset); a signed element index is widened and
+    // scaled into a register pair per load.
     __device__ __forceinline__ void fetch(const float *xs, Buf &v) const {
 #pragma unroll
         for (int e = 0; e < RPT; ++e) {
-            const float *p = xs + goff[e];
+            const char *base = reinterpret_cast<const char *>(xs);
+            const unsigned at = 4u * (unsigned)goff[e];
+            const float *p = reinterpret_cast<const float *>(base + at);
             float c[HC];
             load_cells<HC>(p, c);
-            const float end = p[edge[e]];
+            const float end = *reinterpret_cast<const float *>(base + (at + 4u * (unsigned)edge[e]));
             // lay the values out in window order for either half
 #pragma unroll
             for (int q = 0; q < HC; ++q) v[e][q] = c[q];
@@ -471,6 +477,29 @@ __device__ __forceinline__ void stencil(const float *win, int row00, const float
 #pragma unroll
                 for (int c = 0; c < CPT; ++c) u[c] = fmaf(w[r * 3 + cc][c], v[c + cc], u[c]);
         });
+    }
+}
+
+// Commit R x C gradient values to base[index(r, c)] for the entries with ok(r, c).  One code path
+// per mode (the mode is uniform).  In the add-in-place mode the accumulators were STARTED from
+// the old contents (see the kernels' set-up), so that mode stores like the overwrite mode: an
+// old value fetched at the end instead would put a serial trip to memory at the tail of every
+// workgroup, where nothing is left to hide it.
+template <int R, int C, typename Index, typename Ok>
+__device__ __forceinline__ void commit_grads(float *base, const float (&val)[R][C], int mode,
+                                             Index &&index, Ok &&ok) {
+    if (mode != kParamAtomic) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+                if (ok(r, c)) base[index(r, c)] = val[r][c];
+    } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int c = 0; c < C; ++c)
+                if (ok(r, c)) unsafeAtomicAdd(base + index(r, c), val[r][c]);
     }
 }
 

@@ -36,6 +36,13 @@ struct LnFold {
     const float *g_prev;  // [B,M,N,K] or null
     float *g_out;         // [B,M,N,K] or null
     const float *g_rows;  // [B,M,N,K] G' for the cross-block kernel: g_out, or dy when given
+    // The backward of a chain (chain_bwd.hip) hands what crosses a block boundary to the backward
+    // of the step BEFORE it instead of completing dx itself: per (element, block) the 488
+    // values that the cells around the block receive from it, filed per RECEIVING block
+    // ([B, nblk, 488], see chain_bwd.hip).  halo_in: what the step after left for this one (null:
+    // dy is complete); halo_out: where this step leaves its own (null: dx is completed here).
+    const float *halo_in;
+    float *halo_out;
 };
 
 struct StepArgs {
@@ -84,6 +91,16 @@ int step_backward_fast(const StepArgs &a, hipStream_t st);
 int step_fast_forward_parts(int block_size);   // (mean, M2) pairs, each over forward_part_count cells
 int step_fast_forward_part_count(int block_size);
 int step_fast_backward_parts(int block_size);  // (sum g, sum g*xhat) pairs
+
+// step_fast.hip: the cross-block kernel alone (8^3 blocks, folded LayerNorm arguments in a.ln, the
+// D tensor in a.workspace), for chain_bwd.hip
+int step_cross_launch(const StepArgs &a, int nchunk, int chunk_len, hipStream_t st);
+
+// chain_bwd.hip: backward of one step of a chain with the cross-block part deferred to the step
+// before (a.ln.halo_in / halo_out); fp32, 8^3 blocks, 1..4 inner iterations, normalize off
+bool chain_supports(const StepArgs &a);
+size_t chain_halo_floats(const StepArgs &a);
+int chain_backward(const StepArgs &a, hipStream_t st);
 
 // step_fast.hip: the cross-block kernel on two weight sets, for gated_fast.hip
 int gated_cross_launch(const StepArgs &a, const float *dsum, int nchunk, int chunk_len, hipStream_t st);

@@ -590,29 +590,6 @@ template <int BS, int CPT, int NSLOT> size_t bwd_lds_bytes(int inner, bool ln = 
     return run > setup ? run : setup;
 }
 
-// Commit R x C gradient values to base[index(r, c)] for the entries with ok(r, c).  One code path
-// per mode (the mode is uniform).  In the add-in-place mode the accumulators were STARTED from
-// the old contents (see the kernels' set-up), so that mode stores like the overwrite mode: an
-// old value fetched at the end instead would put a serial trip to memory at the tail of every
-// workgroup, where nothing is left to hide it.
-template <int R, int C, typename Index, typename Ok>
-__device__ __forceinline__ void commit_grads(float *base, const float (&val)[R][C], int mode,
-                                             Index &&index, Ok &&ok) {
-    if (mode != kParamAtomic) {
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int c = 0; c < C; ++c)
-                if (ok(r, c)) base[index(r, c)] = val[r][c];
-    } else {
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-#pragma unroll
-            for (int c = 0; c < C; ++c)
-                if (ok(r, c)) unsafeAtomicAdd(base + index(r, c), val[r][c]);
-    }
-}
-
 // RES (with LN): the outer_residual form of the loop, see LnFold.
 // NORM: per-window normalisation (see step_fwd_fast).  With mean_i, std_i, inv_i = 1/(std_i+eps)
 // of the window before iteration i, n_i = (x_i - mean_i) inv_i what the stencil reads, and
@@ -1613,6 +1590,17 @@ template <bool BWD> int dispatch(const StepArgs &a, hipStream_t st) {
 }
 
 }  // namespace
+
+// The cross-block kernel alone, completing a dx whose block-local part another kernel wrote
+// (8^3 blocks; the LayerNorm fold as a.ln says; D in a.workspace).
+int step_cross_launch(const StepArgs &a, int nchunk, int chunk_len, hipStream_t st) {
+    const int nblk = (a.M / 8) * (a.N / 8) * (a.K / 8);
+    hipLaunchKernelGGL((step_bwd_cross<8, kCrossSlots8, kCrossElems8, true>), dim3(padded_grid(nblk, nchunk)),
+                       dim3(6 * 64 * kCrossSlots8), 0, st, (const float *)a.weight, (const float *)a.x,
+                       (const float *)a.workspace, (float *)a.dx, a.B, a.M, a.N, a.K, nblk, nchunk,
+                       chunk_len, a.ln, (const float *)nullptr);
+    return check_launch("step_bwd_cross");
+}
 
 // The cross-block kernel for the gated update: D0 and D1 of every cell behind one another in
 // `dsum`, weight [27, 2, M, N, K]; same blocks and batch chunks as the kernel that left them.

@@ -43,6 +43,9 @@ EXPORTS = (
     "gridnet_hip_layernorm_backward_sums",
     "gridnet_hip_fused_backward",
     "gridnet_hip_fused_backward_residual",
+    "gridnet_hip_chain_supported",
+    "gridnet_hip_chain_halo_floats",
+    "gridnet_hip_chain_backward",
 )
 
 
@@ -101,6 +104,12 @@ def _load():
     lib.gridnet_hip_fused_backward.argtypes = [i] + [p] * 18 + [i] * 8 + [p, z, p]
     lib.gridnet_hip_fused_backward_residual.restype = i
     lib.gridnet_hip_fused_backward_residual.argtypes = [i] + [p] * 20 + [i] * 8 + [p, z, p]
+    lib.gridnet_hip_chain_supported.restype = i
+    lib.gridnet_hip_chain_supported.argtypes = [i, i, i, i]
+    lib.gridnet_hip_chain_halo_floats.restype = z
+    lib.gridnet_hip_chain_halo_floats.argtypes = [i, i, i, i, i]
+    lib.gridnet_hip_chain_backward.restype = i
+    lib.gridnet_hip_chain_backward.argtypes = [i] + [p] * 20 + [i] * 8 + [p, z, p]
     return lib
 
 

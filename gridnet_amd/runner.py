@@ -10,6 +10,12 @@ step kernels: a step reads the raw output of the step before it and normalises i
 loading, so the LayerNorm costs no pass over the activations of its own (one, for the final
 output).  Same results within rounding; fp32, ``normalize=False``, ``inner >= 1`` only.
 
+With ``fused=True`` and a problem it covers (float32, 8^3 blocks, up to 4 inner iterations) the
+backward of a chain goes through ``gridnet_hip_chain_backward``
+(``chain=True``, the default): the backward hands what crosses a block boundary from step to
+step instead of finishing every dx (one kernel per step instead of two).  Same results to
+rounding.
+
 ``outer_residual=True`` is the other shape of the loop, ``n = norm(h); h = h + (net(n) - n)``
 (gridnet/scripts/train_imagenet.py:81-83), through the fused entry points made for it
 (``fused=True`` only).
@@ -24,7 +30,7 @@ class BodyRunner:
     def __init__(self, weight, bias, scale, gamma, beta, batch: int, inner: int, outer: int,
                  block_size: int, activation: str = "leaky_relu", normalize: bool = False,
                  eps: float = 1e-5, ln_eps: float = 1e-5, backward: bool = True,
-                 fused: bool = False, outer_residual: bool = False):
+                 fused: bool = False, outer_residual: bool = False, chain: bool = True):
         self.w, self.b, self.r, self.gamma, self.beta = weight, bias, scale, gamma, beta
         self.B, (self.M, self.N, self.K) = batch, bias.shape
         if outer < 1:
@@ -85,6 +91,13 @@ class BodyRunner:
                 self.fb_ws_bytes = _n.lib.gridnet_hip_fused_workspace_bytes(
                     batch, self.M, self.N, self.K, inner, block_size, 1)
                 self.fb_ws = _n.workspace(self.fb_ws_bytes, dev)
+        self.chain = bool(chain and fused and backward and not outer_residual and
+                          _n.lib.gridnet_hip_chain_supported(self.dt, inner, block_size, self.normalize))
+        if self.chain:
+            # two buffers that the backward calls of neighbouring steps hand their cross-block
+            # values over in
+            nfl = _n.lib.gridnet_hip_chain_halo_floats(batch, self.M, self.N, self.K, block_size)
+            self.halo = [torch.empty(nfl, device=dev, dtype=dtype) for _ in range(2 if outer > 1 else 0)]
 
     def _mark(self, name, phase):
         if self.on_launch is not None:
@@ -212,6 +225,24 @@ class BodyRunner:
             x = self.s[j - 1] if j else self.x0
             dst = self.ga if g is not self.ga else self.gb
             self._mark("step_bwd", 0)
+            if self.chain:
+                # dx of every step but the first stays unfinished: what crosses a block boundary
+                # travels in halo[j % 2] to the call for step j - 1
+                _n.check(_n.lib.gridnet_hip_chain_backward(
+                    self.dt, self.w.data_ptr(), self.b.data_ptr(), self.r.data_ptr(),
+                    self.gamma.data_ptr(), self.beta.data_ptr(), x.data_ptr(),
+                    self.stats[j - 1].data_ptr() if j else None, g.data_ptr(), self.s[j].data_ptr(),
+                    self.stats[j].data_ptr(), self.sums[j].data_ptr(),
+                    None if j == last else self.halo[(j + 1) % 2].data_ptr(),
+                    self.halo[j % 2].data_ptr() if j else None,
+                    self.dw.data_ptr(), self.db.data_ptr(), self.dr.data_ptr(),
+                    self.dgamma.data_ptr(), self.dbeta.data_ptr(), dst.data_ptr(),
+                    self.sums[j - 1].data_ptr() if j else None, self.B, self.M, self.N, self.K,
+                    self.inner, self.bs, self.act, _n.OVERWRITE_PARAMS if j == last else 0,
+                    self.fb_ws.data_ptr(), self.fb_ws_bytes, stream))
+                self._mark("step_bwd", 1)
+                g = dst
+                continue
             _n.check(_n.lib.gridnet_hip_fused_backward(
                 self.dt, self.w.data_ptr(), self.b.data_ptr(), self.r.data_ptr(),
                 self.gamma.data_ptr(), self.beta.data_ptr(), x.data_ptr(),

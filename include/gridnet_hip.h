@@ -257,6 +257,39 @@ int gridnet_hip_fused_backward_residual(int dtype, const void *weight, const voi
                                         int block_size, int activation, int flags, void *workspace,
                                         size_t workspace_bytes, void *stream);
 
+/*
+ * ---- The backward of a chain that hands gradients across block boundaries from step to step --
+ * gridnet_hip_fused_backward with one change that a caller who runs the whole chain can afford
+ * (no counterpart in the reference, which scatters across block boundaries with global atomics,
+ * src/gridnet_cuda_kernels.cu:424-435): a call may leave dx UNFINISHED.  What the cells of other
+ * blocks receive (one cell deep around every block) is not added to dx but filed, 488 floats per
+ * (element, block), in halo_out [B, nblk, 488]; the call for the step BEFORE takes that buffer as
+ * its halo_in and adds the values while it loads its incoming gradient.  One kernel per step
+ * instead of two, and no scratch tensor written and read back.
+ * float32, normalize = false, block_size 8, 1 <= inner <= 4; gridnet_hip_chain_supported() tells,
+ * other problems use gridnet_hip_fused_backward.  Results agree with it to rounding.
+ */
+int gridnet_hip_chain_supported(int dtype, int inner, int block_size, int normalize);
+
+/* floats of one halo buffer: B * nblk * 488 */
+size_t gridnet_hip_chain_halo_floats(int B, int M, int N, int K, int block_size);
+
+/*   halo_in  == NULL: dy is complete (the last step of a chain);
+ *            != NULL: dy lacks what the call for the step after left there;
+ *   halo_out != NULL: dx receives the block-local part only and halo_out the rest; x_stats and
+ *                     x_sums are required (x_sums is complete: the sums do not wait for dx);
+ *            == NULL: dx is finished here (the first step of a chain), as by
+ *                     gridnet_hip_fused_backward.
+ * Workspace: gridnet_hip_fused_workspace_bytes(.., 1).  Everything else as gridnet_hip_fused_backward. */
+int gridnet_hip_chain_backward(int dtype, const void *weight, const void *bias, const void *scale,
+                               const void *gamma, const void *beta, const void *x,
+                               const void *x_stats, const void *dy, const void *y_raw,
+                               const void *y_stats, const void *y_sums, const void *halo_in,
+                               void *halo_out, void *dweight, void *dbias, void *dscale, void *dgamma,
+                               void *dbeta, void *dx, void *x_sums, int B, int M, int N, int K,
+                               int inner, int block_size, int activation, int flags, void *workspace,
+                               size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -227,6 +227,80 @@ def test_fused_full_size_agrees_with_op_by_op_chain():
         assert torch.equal(a, e), f"{name_}: fused chain is not bitwise reproducible"
 
 
+@pytest.mark.parametrize("shape,batch,inner,outer,activation", [
+    ((16, 16, 16), 3, 1, 3, "silu"),       # 8 blocks: batch split over workgroups, atomics
+    ((8, 24, 16), 5, 2, 2, "tanh"),        # non-cubic, a single block along M (no neighbour there)
+    ((24, 8, 8), 1, 3, 4, "silu"),         # one sample, blocks in a row
+    ((16, 32, 24), 7, 4, 3, "silu"),
+    ((64, 64, 64), 2, 4, 3, "leaky_relu"), # 512 blocks: one workgroup per block, plain stores
+    ((8, 8, 8), 4, 2, 3, "relu"),          # a single block: nothing crosses a boundary
+    ((16, 16, 16), 2, 4, 1, "silu"),       # one outer step: the call that finishes dx itself
+])
+def test_chain_backward_matches_fused_backward(shape, batch, inner, outer, activation):
+    """gridnet_hip_chain_backward (what crosses a block boundary travels from step to step, dx of
+    every step but the first stays unfinished) against gridnet_hip_fused_backward (every dx
+    finished by the cross-block kernel): the same chain both ways, and against the oracle where it
+    finishes in seconds."""
+    from gridnet_amd.runner import BodyRunner
+    from helpers import KINKED, make_acts, make_params
+
+    print(f"chain vs fused backward shape={shape} B={batch} inner={inner} outer={outer} act={activation}",
+          flush=True)
+    w, b, r = make_params(shape, seed=61)
+    g = torch.Generator().manual_seed(62)
+    gamma = 1 + 0.2 * torch.randn(shape, generator=g)
+    beta = 0.2 * torch.randn(shape, generator=g)
+    x0, gy = make_acts(batch, shape, seed=63), make_acts(batch, shape, seed=64)
+    results = []
+    for chain in (False, True):
+        run = BodyRunner(*(v.to(DEV) for v in (w, b, r, gamma, beta)), batch, inner, outer, 8, activation,
+                         False, backward=True, fused=True, chain=chain)
+        assert run.chain == chain
+        y = run.forward(x0.to(DEV)).clone()
+        results.append((y, *[v.clone() for v in run.backward(gy.to(DEV))]))
+    big = shape[0] * shape[1] * shape[2] * batch * inner * outer > 300_000
+    # two fp32 evaluations in different orders: twice the bar between them; under relu /
+    # leaky_relu on millions of cells a few pre-activations sit on the kink, where the order of
+    # evaluation decides the branch: the forward result (continuous) is compared there
+    kinked_and_big = activation in KINKED and big
+    for name_, a, e in zip(NAMES, results[1], results[0]):
+        if name_ == "y":
+            assert torch.equal(a, e), "the forward is the same kernel"
+        elif not kinked_and_big:
+            assert_close(a, e.double().cpu(), rtol=2e-4, atol=2e-5, what=name_)
+    if not big:
+        exp = network_forward_backward([v.double() for v in (w, b, r, gamma, beta)], x0.double(), gy.double(),
+                                       inner_iterations=inner, outer_iterations=outer, block_size=8,
+                                       activation=activation, normalize=False)
+        if activation not in KINKED:
+            for name_, a, e in zip(NAMES, results[1], exp):
+                assert_close(a, e, what=name_)
+
+
+def test_chain_entry_point_rejects_what_it_does_not_cover():
+    from gridnet_amd import native as n
+
+    assert n.lib.gridnet_hip_chain_supported(n.F32, 4, 8, 0) == 1
+    assert n.lib.gridnet_hip_chain_supported(n.F32, 5, 8, 0) == 0   # the LDS holds 4 iterations
+    assert n.lib.gridnet_hip_chain_supported(n.F32, 4, 4, 0) == 0   # 8^3 blocks only
+    assert n.lib.gridnet_hip_chain_supported(n.F64, 4, 8, 0) == 0
+    assert n.lib.gridnet_hip_chain_supported(n.F32, 4, 8, 1) == 0
+    assert n.lib.gridnet_hip_chain_halo_floats(32, 64, 64, 64, 8) == 32 * 512 * 488
+    x = torch.zeros(1, 8, 8, 8, device=DEV)
+    p = x.data_ptr()
+    args = [p] * 11
+    # halo_out without x_stats: an unfinished dx is for a step whose input passes a LayerNorm
+    rc = n.lib.gridnet_hip_chain_backward(n.F32, p, p, p, p, p, p, None, p, p, p, p, None, p, p, p, p, p, p,
+                                          p, None, 1, 8, 8, 8, 2, 8, 2, 0, p, 1 << 20, n.current_stream(x))
+    assert rc != 0 and "halo_out" in n.last_error()
+    rc = n.lib.gridnet_hip_chain_backward(n.F32, p, p, p, p, p, p, None, p, p, p, p, None, None, p, p, p, p, p,
+                                          p, None, 1, 8, 8, 8, 5, 8, 2, 0, p, 1 << 20, n.current_stream(x))
+    assert rc != 0 and "inner" in n.last_error()
+    rc = n.lib.gridnet_hip_chain_backward(n.F32, p, p, p, p, p, p, None, p, p, p, p, None, None, p, p, p, p, p,
+                                          p, None, 1, 8, 8, 8, 2, 8, 2, 0, p, 0, n.current_stream(x))
+    assert rc != 0 and "workspace" in n.last_error()
+
+
 def test_fused_rejects_what_it_does_not_cover():
     from gridnet_amd import native as n
 
