@@ -155,7 +155,7 @@ void step_fwd_fast(
                         make_float4(part[0], part[1], part[2], part[3]);
             } else fx.commit(win, pre);
         }
-        lds_barrier();
+        slot_barrier<TL::TPS>();
         if (done_s >= 0) {
             if (NORM) {
 #pragma unroll
@@ -220,7 +220,7 @@ void step_fwd_fast(
                             make_float2(s1, s2);
                 }
             }
-            lds_barrier();
+            slot_barrier<TL::TPS>();
         }
         if (RES && active) {
 #pragma unroll
@@ -250,7 +250,7 @@ void step_fwd_fast(
         done_shift = shift;
 #pragma unroll
         for (int c = 0; c < CPT; ++c) done[c] = cur[c];
-        if (inner == 0) lds_barrier();  // `cur` was read from the window that is rewritten next
+        if (inner == 0) slot_barrier<TL::TPS>();  // `cur` was read from the window that is rewritten next
     }
     if (done_s >= 0) {
         if (NORM) {
@@ -845,7 +845,7 @@ void step_bwd_fast(
         const int s = sb + pl.slot;
         const bool active = s < s1;  // a slot past the end idles through the barriers
         take_turns(sb / NSLOT);
-        lds_barrier();               // this element's window
+        slot_barrier<TL::TPS>();               // this element's window
         finish_done();
         if (s + NSLOT < s1) fetch_element(s + NSLOT);
         float cur[CPT];
@@ -916,7 +916,7 @@ void step_bwd_fast(
                     for (int c = 0; c < CPT; ++c) win[((it + 1) & 1) * TL::WIN + pl.own + c] = 0.f;
                 }
             }
-            if (it + 1 < inner) lds_barrier();
+            if (it + 1 < inner) slot_barrier<TL::TPS>();
         }
 
         // ---- reverse sweep: delta window copy (it & 1) holds delta_it ----
@@ -959,7 +959,7 @@ void step_bwd_fast(
                 // iteration's barrier, so that nobody commits the next element's window while
                 // the halo is read; behind a barrier of its own when the zeros of the halo
                 // window were written in the iteration just before (inner == 1).
-                if (inner == 1) lds_barrier();
+                if (inner == 1) slot_barrier<TL::TPS>();
                 if (active)
                     for_each_row<TL, CPT, kBwdDepth>(xhalo + pl.row00, [&](int r, const float (&xv)[CPT + 2]) {
 #pragma unroll
@@ -969,7 +969,7 @@ void step_bwd_fast(
                                 nw[r * 3 + cc][c] = fmaf(xv[c + cc], dsum[c], nw[r * 3 + cc][c]);
                     });
             }
-            lds_barrier();
+            slot_barrier<TL::TPS>();
             if (NORM && active && it == inner - 1) {
                 // once per element: what the owned cells' taps into the halo see there (the
                 // halo window holds zeros in the block's cells, so the other taps add nothing)
@@ -1031,7 +1031,7 @@ void step_bwd_fast(
             }
         }
 
-        if (inner == 0) lds_barrier();  // no barrier since the top: others may still read LDS
+        if (inner == 0) slot_barrier<TL::TPS>();  // no barrier since the top: others may still read LDS
         done_s = active ? s : -1;
 #pragma unroll
         for (int c = 0; c < CPT; ++c) {
