@@ -90,8 +90,6 @@ class ImageNetGridModel(nn.Module):
         super().__init__()
         assert 256 % grid_size == 0
         # not in the reference: run the loop as one autograd node on the fused entry points
-        if fused_body and separate_params:
-            raise ValueError("the fused body shares its parameters between the outer iterations")
         self.fused_body = fused_body
         self.outer_iters = outer_iters
         self.outer_residual = outer_residual
@@ -122,8 +120,8 @@ class ImageNetGridModel(nn.Module):
     def forward(self, images: torch.Tensor) -> torch.Tensor:
         h = self.embed(images)
         if self.fused_body:
-            return self.readout(fused_body(h, self.network, self.norm, self.outer_iters,
-                                           self.outer_residual))
+            return self.readout(fused_body(h, self.networks if self.separate_params else self.network,
+                                           self.norm, self.outer_iters, self.outer_residual))
         for i in range(self.outer_iters):
             net = self.networks[i] if self.separate_params else self.network
             if self.outer_residual:

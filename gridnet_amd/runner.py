@@ -16,6 +16,10 @@ backward of a chain goes through ``gridnet_hip_chain_backward``
 step instead of finishing every dx (one kernel per step instead of two).  Same results to
 rounding.
 
+``weight``, ``bias`` and ``scale`` may each be a list of ``outer`` tensors: one parameter set
+per outer step (the reference's ``--separate_params``, gridnet/scripts/train_imagenet.py:54-58).
+``backward`` then returns lists of gradients for them, one entry per step.
+
 ``outer_residual=True`` is the other shape of the loop, ``n = norm(h); h = h + (net(n) - n)``
 (gridnet/scripts/train_imagenet.py:81-83), through the fused entry points made for it
 (``fused=True`` only).
@@ -31,6 +35,14 @@ class BodyRunner:
                  block_size: int, activation: str = "leaky_relu", normalize: bool = False,
                  eps: float = 1e-5, ln_eps: float = 1e-5, backward: bool = True,
                  fused: bool = False, outer_residual: bool = False, chain: bool = True):
+        self.separate = isinstance(weight, (list, tuple))
+        if self.separate:
+            if not (len(weight) == len(bias) == len(scale) == outer):
+                raise ValueError("separate parameters: one weight, bias and scale per outer step")
+            self.ws, self.bs_, self.rs = list(weight), list(bias), list(scale)
+        else:
+            self.ws, self.bs_, self.rs = [weight] * max(outer, 1), [bias] * max(outer, 1), [scale] * max(outer, 1)
+        weight, bias, scale = self.ws[0], self.bs_[0], self.rs[0]
         self.w, self.b, self.r, self.gamma, self.beta = weight, bias, scale, gamma, beta
         self.B, (self.M, self.N, self.K) = batch, bias.shape
         if outer < 1:
@@ -65,9 +77,14 @@ class BodyRunner:
         if backward:
             self.ga = torch.empty(shape, device=dev, dtype=dtype)
             self.gb = torch.empty(shape, device=dev, dtype=dtype)
-            self.dw = torch.empty_like(weight)
-            self.db = torch.empty_like(bias)
-            self.dr = torch.empty_like(bias)
+            # one gradient set per parameter set.  The entry points either overwrite all parameter
+            # gradients of a call or accumulate into all of them, the LayerNorm's (shared by the
+            # steps) included: with separate parameters the last step's call overwrites, the
+            # others accumulate into buffers that backward() zero-fills first
+            n_sets = outer if self.separate else 1
+            self.dw_all = torch.empty((n_sets,) + tuple(weight.shape), device=dev, dtype=dtype)
+            self.db_all = torch.empty((n_sets,) + tuple(bias.shape), device=dev, dtype=dtype)
+            self.dr_all = torch.empty((n_sets,) + tuple(bias.shape), device=dev, dtype=dtype)
             self.dgamma = torch.empty_like(bias)
             self.dbeta = torch.empty_like(bias)
             self.bw_ws_bytes = _n.lib.gridnet_hip_backward_workspace_bytes(
@@ -99,14 +116,34 @@ class BodyRunner:
             nfl = _n.lib.gridnet_hip_chain_halo_floats(batch, self.M, self.N, self.K, block_size)
             self.halo = [torch.empty(nfl, device=dev, dtype=dtype) for _ in range(2 if outer > 1 else 0)]
 
+    def _params(self, j):
+        """Device pointers of the parameter set of outer step j."""
+        return self.ws[j].data_ptr(), self.bs_[j].data_ptr(), self.rs[j].data_ptr()
+
+    def _grads(self, j):
+        """Device pointers of the gradient buffers that outer step j accumulates into."""
+        k = j if self.separate else 0
+        return self.dw_all[k].data_ptr(), self.db_all[k].data_ptr(), self.dr_all[k].data_ptr()
+
+    def _param_grads(self):
+        if self.separate:
+            return list(self.dw_all), list(self.db_all), list(self.dr_all)
+        return self.dw_all[0], self.db_all[0], self.dr_all[0]
+
+    def _zero_separate_grads(self):
+        if self.separate and self.outer > 1:
+            self.dw_all[:-1].zero_()
+            self.db_all[:-1].zero_()
+            self.dr_all[:-1].zero_()
+
     def _mark(self, name, phase):
         if self.on_launch is not None:
             self.on_launch(name, phase)
 
-    def step_forward(self, x, y, stream):
+    def step_forward(self, x, y, stream, j=0):
         self._mark("step_fwd", 0)
         _n.check(_n.lib.gridnet_hip_forward(
-            self.dt, self.w.data_ptr(), self.b.data_ptr(), self.r.data_ptr(), x.data_ptr(),
+            self.dt, *self._params(j), x.data_ptr(),
             y.data_ptr(), self.B, self.M, self.N, self.K, self.inner, self.bs, self.eps,
             self.normalize, self.act, stream))
         self._mark("step_fwd", 1)
@@ -131,7 +168,7 @@ class BodyRunner:
             y_stats = self.stats[j if keep else j % 2]
             self._mark("step_fwd", 0)
             _n.check(_n.lib.gridnet_hip_fused_forward(
-                self.dt, self.w.data_ptr(), self.b.data_ptr(), self.r.data_ptr(),
+                self.dt, *self._params(j),
                 self.gamma.data_ptr(), self.beta.data_ptr(), x.data_ptr(),
                 x_stats.data_ptr() if x_stats is not None else None, y.data_ptr(),
                 y_stats.data_ptr(), self.B, self.M, self.N, self.K, self.inner, self.bs,
@@ -162,7 +199,7 @@ class BodyRunner:
             out_stats = self.stats[j + 1 if keep else (j + 1) % 2]
             self._mark("step_fwd", 0)
             _n.check(_n.lib.gridnet_hip_fused_forward_residual(
-                self.dt, self.w.data_ptr(), self.b.data_ptr(), self.r.data_ptr(),
+                self.dt, *self._params(j),
                 self.gamma.data_ptr(), self.beta.data_ptr(), h.data_ptr(), stats.data_ptr(),
                 out.data_ptr(), out_stats.data_ptr(), self.B, self.M, self.N, self.K, self.inner,
                 self.bs, self.ln_eps, self.act, self.fw_ws.data_ptr(), self.fw_ws_bytes, stream))
@@ -187,7 +224,7 @@ class BodyRunner:
             x = self.h[j] if j else self.x0
             self._mark("step_bwd", 0)
             _n.check(_n.lib.gridnet_hip_fused_backward_residual(
-                self.dt, self.w.data_ptr(), self.b.data_ptr(), self.r.data_ptr(),
+                self.dt, *self._params(j),
                 self.gamma.data_ptr(), self.beta.data_ptr(), x.data_ptr(), self.stats[j].data_ptr(),
                 (grad_out if given else dn[(j + 1) % 2]).data_ptr(),
                 None if given else self.h[j + 1].data_ptr(),
@@ -195,7 +232,7 @@ class BodyRunner:
                 None if given else self.sums[j + 1].data_ptr(),
                 None if given else grad_wrt(j + 2).data_ptr(),
                 None if given else grad_wrt(j + 1).data_ptr(),
-                self.dw.data_ptr(), self.db.data_ptr(), self.dr.data_ptr(), self.dgamma.data_ptr(),
+                *self._grads(j), self.dgamma.data_ptr(),
                 self.dbeta.data_ptr(), dn[j % 2].data_ptr(), self.sums[j].data_ptr(),
                 self.B, self.M, self.N, self.K, self.inner, self.bs, self.act,
                 _n.OVERWRITE_PARAMS if given else 0, self.fb_ws.data_ptr(), self.fb_ws_bytes, stream))
@@ -209,7 +246,7 @@ class BodyRunner:
             self.ln_ws.data_ptr(), self.ln_ws_bytes, stream))
         self._mark("ln_bwd", 1)
         torch.add(dn[1], grad_wrt(1), out=dn[1])
-        return self.dw, self.db, self.dr, self.dgamma, self.dbeta, dn[1]
+        return (*self._param_grads(), self.dgamma, self.dbeta, dn[1])
 
     def _fused_backward(self, grad_out):
         stream = _n.current_stream(self.w)
@@ -229,14 +266,13 @@ class BodyRunner:
                 # dx of every step but the first stays unfinished: what crosses a block boundary
                 # travels in halo[j % 2] to the call for step j - 1
                 _n.check(_n.lib.gridnet_hip_chain_backward(
-                    self.dt, self.w.data_ptr(), self.b.data_ptr(), self.r.data_ptr(),
+                    self.dt, *self._params(j),
                     self.gamma.data_ptr(), self.beta.data_ptr(), x.data_ptr(),
                     self.stats[j - 1].data_ptr() if j else None, g.data_ptr(), self.s[j].data_ptr(),
                     self.stats[j].data_ptr(), self.sums[j].data_ptr(),
                     None if j == last else self.halo[(j + 1) % 2].data_ptr(),
                     self.halo[j % 2].data_ptr() if j else None,
-                    self.dw.data_ptr(), self.db.data_ptr(), self.dr.data_ptr(),
-                    self.dgamma.data_ptr(), self.dbeta.data_ptr(), dst.data_ptr(),
+                    *self._grads(j), self.dgamma.data_ptr(), self.dbeta.data_ptr(), dst.data_ptr(),
                     self.sums[j - 1].data_ptr() if j else None, self.B, self.M, self.N, self.K,
                     self.inner, self.bs, self.act, _n.OVERWRITE_PARAMS if j == last else 0,
                     self.fb_ws.data_ptr(), self.fb_ws_bytes, stream))
@@ -244,18 +280,17 @@ class BodyRunner:
                 g = dst
                 continue
             _n.check(_n.lib.gridnet_hip_fused_backward(
-                self.dt, self.w.data_ptr(), self.b.data_ptr(), self.r.data_ptr(),
+                self.dt, *self._params(j),
                 self.gamma.data_ptr(), self.beta.data_ptr(), x.data_ptr(),
                 self.stats[j - 1].data_ptr() if j else None, g.data_ptr(), self.s[j].data_ptr(),
-                self.stats[j].data_ptr(), self.sums[j].data_ptr(), self.dw.data_ptr(),
-                self.db.data_ptr(), self.dr.data_ptr(), self.dgamma.data_ptr(),
+                self.stats[j].data_ptr(), self.sums[j].data_ptr(), *self._grads(j), self.dgamma.data_ptr(),
                 self.dbeta.data_ptr(), dst.data_ptr(), self.sums[j - 1].data_ptr() if j else None,
                 self.B, self.M, self.N, self.K, self.inner, self.bs, self.act,
                 _n.OVERWRITE_PARAMS if j == last else 0, self.fb_ws.data_ptr(), self.fb_ws_bytes,
                 stream))
             self._mark("step_bwd", 1)
             g = dst
-        return self.dw, self.db, self.dr, self.dgamma, self.dbeta, g
+        return (*self._param_grads(), self.dgamma, self.dbeta, g)
 
     def forward(self, x0):
         """Returns the buffer holding the result (valid until the next call)."""
@@ -267,11 +302,11 @@ class BodyRunner:
         self.x0 = x0  # read in place (and again by backward): the caller keeps it unchanged
         if self.has_backward:
             for j in range(self.outer):
-                self.step_forward(self.h[j] if j else x0, self.s[j], stream)
+                self.step_forward(self.h[j] if j else x0, self.s[j], stream, j)
                 self.norm_forward(self.s[j], self.h[j + 1], j, stream)
             return self.h[self.outer]
         for j in range(self.outer):  # forward only: ping-pong, nothing is kept
-            self.step_forward(self.h[j % 2] if j else x0, self.s[0], stream)
+            self.step_forward(self.h[j % 2] if j else x0, self.s[0], stream, j)
             self.norm_forward(self.s[0], self.h[(j + 1) % 2], 0, stream)
         return self.h[self.outer % 2]
 
@@ -279,6 +314,7 @@ class BodyRunner:
         """Backward of the last ``forward``.  Returns (dweight, dbias, dscale, dgamma, dbeta, dx0);
         parameter gradients are summed over the outer steps (shared parameters)."""
         assert self.has_backward
+        self._zero_separate_grads()
         if self.outer_residual:
             return self._residual_backward(grad_out)
         if self.fused:
@@ -298,12 +334,11 @@ class BodyRunner:
             # dx is fully written every time; parameter gradients are written by the first
             # call and accumulated into by the later ones (parameters are shared)
             _n.check(_n.lib.gridnet_hip_backward(
-                self.dt, self.w.data_ptr(), self.b.data_ptr(), self.r.data_ptr(),
-                (self.h[j] if j else self.x0).data_ptr(), self.ga.data_ptr(), self.dw.data_ptr(),
-                self.db.data_ptr(),
-                self.dr.data_ptr(), self.gb.data_ptr(), self.B, self.M, self.N, self.K, self.inner,
+                self.dt, *self._params(j),
+                (self.h[j] if j else self.x0).data_ptr(), self.ga.data_ptr(), *self._grads(j),
+                self.gb.data_ptr(), self.B, self.M, self.N, self.K, self.inner,
                 self.bs, self.eps, self.normalize, self.act, flags | _n.OVERWRITE_DX,
                 self.bw_ws.data_ptr(), self.bw_ws_bytes, stream))
             self._mark("step_bwd", 1)
             g = self.gb
-        return self.dw, self.db, self.dr, self.dgamma, self.dbeta, self.gb
+        return (*self._param_grads(), self.dgamma, self.dbeta, self.gb)

@@ -258,6 +258,32 @@ def test_models_with_the_fused_body_match_the_reference_loop():
         MnistGridModel(2, 2, 1.0, 1.0, "tanh", True, 0.0, dev, fused_body=True)
 
 
+@pytest.mark.parametrize("outer_residual", [False, True], ids=["plain", "outer_residual"])
+def test_fused_body_with_separate_parameters_per_outer_step(outer_residual):
+    """The reference's --separate_params (gridnet/scripts/train_imagenet.py:54-58, 76-80): one
+    Gridnet per outer iteration.  The fused body takes the list and returns every network's own
+    gradients; held to the op-by-op loop of the same model."""
+    from gridnet_amd.models import ImageNetGridModel
+
+    torch.manual_seed(8)
+    dev = torch.device(DEV)
+    print(f"separate_params outer_residual={outer_residual}", flush=True)
+    kw = dict(inner_iters=2, outer_iters=3, outer_residual=outer_residual, init_scale=1.0,
+              residual_scale=0.5, emb_channels=4, grid_size=16, activation="silu", separate_params=True,
+              device=dev)
+    plain, fused = ImageNetGridModel(**kw), ImageNetGridModel(fused_body=True, **kw)
+    fused.load_state_dict(plain.state_dict())
+    weights = [net.weight for net in plain.networks]
+    assert not torch.equal(weights[0], weights[1]), "the networks must differ for this to test anything"
+    batch = torch.randn(2, 3, 256, 256, device=dev)
+    for m in (plain, fused):
+        m(batch).square().mean().backward()
+    torch.testing.assert_close(fused(batch), plain(batch), rtol=1e-4, atol=1e-5)
+    for (name, p), q in zip(plain.named_parameters(), fused.parameters()):
+        assert q.grad is not None, name
+        torch.testing.assert_close(q.grad, p.grad, rtol=1e-3, atol=1e-5, msg=lambda m, n=name: f"{n}: {m}")
+
+
 def test_two_streams_in_flight_do_not_disturb_each_other():
     """The library keeps no state between calls and launches on the stream it is given: two
     chains enqueued alternately on two streams (their kernels free to overlap on the device)
