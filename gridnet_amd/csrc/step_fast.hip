@@ -560,6 +560,214 @@ void step_fwd_split(
     if (done_s >= 0) store_result(done_s, done);
 }
 
+// ---- forward, 8^3 blocks, the chain's variant: two batch elements per pass -------------------
+// step_fwd_split<ACT, LN = true> with every thread advancing TWO batch elements side by side:
+// the same 108 weights in registers feed both, the two elements' dependent FMA chains and LDS
+// round trips interleave (neither the LDS nor the vector ALU is saturated by one element per
+// wave: what limits step_fwd_split is latency), a barrier serves two elements, and with fewer,
+// larger workgroups the 29 parameter planes of a block are fetched twice per launch instead of
+// three times (64^3 grid, batch 32).  Two waves per SIMD instead of three: the second element's
+// state and prefetch need the registers.
+template <int ACT>
+__global__ __launch_bounds__(128) __attribute__((amdgpu_waves_per_eu(2)))
+void step_fwd_pair(
+    const float *__restrict__ weight, const float *__restrict__ bias,
+    const float *__restrict__ scale, const float *__restrict__ x, float *__restrict__ y, int B, int M,
+    int N, int K, int inner, int nblk, int nchunk, int chunk_len, LnFold ln) {
+    using TL = Tile<8, 4>;
+    using SW = SplitWin;
+    using FX = Fetch<TL>;
+    constexpr int E = 2;
+    // per element two copies of the window; then gamma and beta laid out alike
+    __shared__ __attribute__((aligned(16))) float lds[(2 * E + 2) * SW::COPY];
+    float *gwin = lds + 2 * E * SW::COPY, *bwin = gwin + SW::COPY;
+    const bool ln_in = ln.x_stats != nullptr;  // x is the raw output of the step before
+
+    int blk, chunk;
+    if (!split_block_id(blockIdx.x, nblk, nchunk, blk, chunk)) return;  // grid padding
+    const Place<TL, 4, 1> pl(threadIdx.x, blk, N, K);
+    const FX fx(pl.lane, pl.p0, pl.q0, pl.r0, M, N, K);
+    const long cells = (long)M * N * K;
+    const bool second = pl.kt != 0;  // this thread holds columns 7 6 5 4, in that order
+
+    int cen_at[FX::RPT], side_at[FX::RPT];
+#pragma unroll
+    for (int e = 0; e < FX::RPT; ++e) {
+        const int id = pl.lane + e * TL::TPS;
+        const int half = id & 1, row = id >> 1;
+        const int wj = row % SW::S, wi = row / SW::S;
+        cen_at[e] = wi * SW::PS + wj * SW::RS + half * 4;
+        side_at[e] = SW::CEN + half * SW::SS + wi * SW::SP + wj;
+    }
+    const int cen00 = pl.i * SW::PS + pl.j * SW::RS + pl.kt * 4;
+    const int side00 = SW::CEN + pl.kt * SW::SS + pl.i * SW::SP + pl.j;
+    const int own = cen00 + SW::PS + SW::RS;
+
+    // parameters in register order (see step_fwd_split)
+    float w[27][4], bv[4], rv[4];
+#pragma unroll
+    for (int ab = 0; ab < 9; ++ab) {
+        float wt[3][4];
+#pragma unroll
+        for (int cc = 0; cc < 3; ++cc) load_cells<4>(weight + (ab * 3 + cc) * cells + pl.gc, wt[cc]);
+#pragma unroll
+        for (int cc = 0; cc < 3; ++cc)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) w[ab * 3 + cc][r] = second ? wt[2 - cc][3 - r] : wt[cc][r];
+    }
+    {
+        float bt[4], rt[4];
+        load_cells<4>(bias + pl.gc, bt);
+        load_cells<4>(scale + pl.gc, rt);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            bv[r] = second ? bt[3 - r] : bt[r];
+            rv[r] = second ? rt[3 - r] : rt[r];
+        }
+    }
+    auto commit = [&](float *to, int copies, const typename FX::Buf &v, bool fold, float mean, float rstd) {
+#pragma unroll
+        for (int e = 0; e < FX::RPT; ++e)
+            if (fx.loff[e] >= 0) {
+                float end = v[e][4], c[4];
+#pragma unroll
+                for (int r = 0; r < 4; ++r) c[r] = fx.hi[e] ? v[e][3 - r] : v[e][r];
+                if (fold) {
+                    const float4 g4 = *reinterpret_cast<const float4 *>(gwin + cen_at[e]);
+                    const float4 b4 = *reinterpret_cast<const float4 *>(bwin + cen_at[e]);
+                    c[0] = fmaf((c[0] - mean) * rstd, g4.x, b4.x);
+                    c[1] = fmaf((c[1] - mean) * rstd, g4.y, b4.y);
+                    c[2] = fmaf((c[2] - mean) * rstd, g4.z, b4.z);
+                    c[3] = fmaf((c[3] - mean) * rstd, g4.w, b4.w);
+                    end = fmaf((end - mean) * rstd, gwin[side_at[e]], bwin[side_at[e]]);
+                }
+                if (!(fx.ok[e] && fx.edge_ok[e])) end = 0.f;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) c[r] = fx.ok[e] ? c[r] : 0.f;
+                for (int copy = 0; copy < copies; ++copy) {
+                    *reinterpret_cast<float4 *>(to + copy * SW::COPY + cen_at[e]) =
+                        make_float4(c[0], c[1], c[2], c[3]);
+                    to[copy * SW::COPY + side_at[e]] = end;
+                }
+            }
+    };
+    typename FX::Buf pre[E];
+    if (ln_in) {  // gamma and beta of the window, once per workgroup
+        fx.fetch(ln.gamma, pre[0]);
+        commit(gwin, 1, pre[0], false, 0.f, 1.f);
+        fx.fetch(ln.beta, pre[0]);
+        commit(bwin, 1, pre[0], false, 0.f, 1.f);
+        lds_barrier();
+    }
+    auto store_result = [&](int s, const float (&cur)[4]) {
+        float out[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) out[c] = second ? cur[3 - c] : cur[c];
+        store_cells<4>(y + s * cells + pl.gc, out);
+    };
+
+    const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
+    float pre_mean[E], pre_rstd[E];
+    // Loads are unconditional: past the end of the chunk they repeat its last element, whose
+    // copy nobody stores (with branches around them the compiler cannot count the loads in flight)
+    auto fetch_pair = [&](int s) {
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const int sc = min(s + e, s1 - 1);
+            fx.fetch(x + sc * cells, pre[e]);
+            pre_mean[e] = ln_in ? load_ahead(ln.x_stats, 2 * sc) : 0.f;
+            pre_rstd[e] = ln_in ? load_ahead(ln.x_stats, 2 * sc + 1) : 1.f;
+        }
+    };
+    if (s0 < s1) fetch_pair(s0);
+    float done[E][4];
+    int done_s = -1;
+    const bool turns = nchunk > 1;
+    for (int s = s0; s < s1; s += E) {
+        if (turns) take_turns(s >> 1);
+#pragma unroll
+        for (int e = 0; e < E; ++e) commit(lds + e * 2 * SW::COPY, 2, pre[e], ln_in, pre_mean[e], pre_rstd[e]);
+        lds_barrier();
+        if (done_s >= 0) {
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+                if (done_s + e < s1) store_result(done_s + e, done[e]);
+        }
+        if (s + E < s1) fetch_pair(s + E);  // next pair, in flight
+        float cur[E][4];
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const float4 q = *reinterpret_cast<const float4 *>(lds + e * 2 * SW::COPY + own);
+            cur[e][0] = q.x; cur[e][1] = q.y; cur[e][2] = q.z; cur[e][3] = q.w;
+        }
+        for (int it = 0; it < inner; ++it) {
+            float u[E][4];
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) u[e][r] = bv[r];
+#pragma unroll
+            for (int a = 0; a < 3; ++a)
+#pragma unroll
+                for (int b = 0; b < 3; ++b) {
+#pragma unroll
+                    for (int e = 0; e < E; ++e) {
+                        const float *from = lds + (e * 2 + (it & 1)) * SW::COPY;
+                        const float4 q =
+                            *reinterpret_cast<const float4 *>(from + cen00 + a * SW::PS + b * SW::RS);
+                        float v[6];
+                        v[0] = from[side00 + a * SW::SP + b];
+                        v[1] = q.x; v[2] = q.y; v[3] = q.z; v[4] = q.w;
+                        v[5] = partner_lane(q.w);
+#pragma unroll
+                        for (int cc = 0; cc < 3; ++cc)
+#pragma unroll
+                            for (int r = 0; r < 4; ++r)
+                                u[e][r] = fmaf(w[a * 9 + b * 3 + cc][r], v[r + cc], u[e][r]);
+                    }
+                }
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) cur[e][r] = fmaf(rv[r], Act<ACT, float>::f(u[e][r]), cur[e][r]);
+                *reinterpret_cast<float4 *>(lds + (e * 2 + ((it + 1) & 1)) * SW::COPY + own) =
+                    make_float4(cur[e][0], cur[e][1], cur[e][2], cur[e][3]);
+            }
+            lds_barrier();
+        }
+        if (ln.y_part) {
+            // statistics of the results for the LayerNorm that follows: one (mean, M2) pair per wave
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+                float sum = 0.f, m2 = 0.f;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) sum += cur[e][r];
+                const float mean = row16_sum(sum) * (1.f / 64);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) m2 = fmaf(cur[e][r] - mean, cur[e][r] - mean, m2);
+                m2 = row16_sum(m2);
+                float wave_mean, wave_m2;
+                slot_wave_moments<128>(mean, m2, 64, wave_mean, wave_m2);
+                if ((pl.lane & 63) == 0 && s + e < s1) {
+                    float *to = ln.y_part + (((long)(s + e) * nblk + blk) * 2 + pl.lane / 64) * 2;
+                    to[0] = wave_mean;
+                    to[1] = wave_m2;
+                }
+            }
+        }
+        done_s = s;
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) done[e][r] = cur[e][r];
+    }
+    if (done_s >= 0) {
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+            if (done_s + e < s1) store_result(done_s + e, done[e]);
+    }
+}
+
 // ---- backward ------------------------------------------------------------------------------
 constexpr int kBwdDepth = 4;  // neighbour rows requested ahead of the arithmetic
 
@@ -1475,6 +1683,21 @@ int launch_fwd_split(const StepArgs &a, hipStream_t st) {
                        p.chunk_len, a.ln, (float)a.eps);
     return check_launch("step_fwd_split");
 }
+template <int ACT> int launch_fwd_pair(const StepArgs &a, hipStream_t st) {
+    auto kern = step_fwd_pair<ACT>;
+    static int per_cu = 0;
+    if (per_cu == 0) {
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, 128, 0) != hipSuccess || n < 1) n = 1;
+        per_cu = n;
+    }
+    const Plan p = make_plan(a, 2, per_cu * device_cus(), false);
+    hipLaunchKernelGGL(kern, dim3(padded_grid(p.nblk, p.nchunk)), dim3(128), 0, st,
+                       (const float *)a.weight, (const float *)a.bias, (const float *)a.scale,
+                       (const float *)a.x, (float *)a.y, a.B, a.M, a.N, a.K, a.inner, p.nblk, p.nchunk,
+                       p.chunk_len, a.ln);
+    return check_launch("step_fwd_pair");
+}
 template <int BS, int CPT, int NSLOT, int ACT> int launch_fwd(const StepArgs &a, hipStream_t st) {
     if (a.normalize) {
         if (BS == 8) return launch_fwd_split<ACT, false, false, true>(a, st);
@@ -1483,6 +1706,17 @@ template <int BS, int CPT, int NSLOT, int ACT> int launch_fwd(const StepArgs &a,
     if (a.ln.gamma && a.ln.residual) {
         if (BS == 8) return launch_fwd_split<ACT, true, true>(a, st);
         return launch_fwd_ln<BS, CPT, NSLOT, ACT, true, true>(a, st);
+    }
+    // The chain's forward on SMALL grids (fewer blocks than a sixth of the workgroups the chip
+    // holds, so that a workgroup of step_fwd_split gets four batch elements or fewer for one fetch
+    // of its 29 parameter planes): two elements per pass.  Measured with 3 waves per SIMD for
+    // step_fwd_split: 32^3 grid, batch 64: 0.279 -> 0.238 ms per 8-step chain; on larger grids the
+    // lower occupancy of the pair kernel costs more than it brings (64^3 / batch 32: 66 -> 69 us
+    // per step, 128^3 / batch 8: 2.61 -> 3.00 ms per 16-step chain).
+    if (BS == 8 && a.ln.gamma && a.B >= 2 && a.inner >= 1) {
+        const int nblk = (a.M / 8) * (a.N / 8) * (a.K / 8);
+        const int chunks = 6 * device_cus() / nblk;  // what step_fwd_split's plan would use
+        if (chunks >= 1 && (a.B + chunks - 1) / chunks <= 4) return launch_fwd_pair<ACT>(a, st);
     }
     if (BS == 8) return a.ln.gamma ? launch_fwd_split<ACT, true>(a, st) : launch_fwd_split<ACT, false>(a, st);
     if (a.ln.gamma) return launch_fwd_ln<BS, CPT, NSLOT, ACT, true>(a, st);
