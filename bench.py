@@ -20,6 +20,11 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor peak
 FP32_PEAK_TFLOPS = 157.3  # MI355X vector fp32, vendor peak (with packed fp32 instructions)
+# This build compiles with packed fp32 arithmetic switched off: one FMA per lane and clock,
+# 256 CUs x 4 SIMDs x 16 lanes x 2 flop x 2.4 GHz = half the vendor figure.
+FP32_UNPACKED_PEAK_TFLOPS = FP32_PEAK_TFLOPS / 2
+LDS_BYTES_PER_CLOCK_PER_CU = 128
+CUS = 256
 
 
 def gpu_run(wl, steps, warmup, fused, graph_replay=True):
@@ -241,15 +246,23 @@ def main():
         bytes_["step_fwd"] += bytes_["ln_fwd"]
         bytes_["step_bwd"] += bytes_["ln_bwd"]
     dominant = max(kernel_s, key=lambda k: kernel_s[k])
-    # HBM bytes per call of that entry point, from the committed rocprofv3 --pmc summary
-    # (FETCH_SIZE and WRITE_SIZE runs, scaled by a copy kernel of known size); null if absent
-    traffic = None
+    # HBM bytes per call of that entry point and the counters of its main kernel, from the
+    # committed rocprofv3 --pmc summaries (FETCH_SIZE and WRITE_SIZE scaled by a copy kernel of
+    # known size); null if absent
+    traffic, counters, counted_kernel = None, {}, None
     try:
-        with open(os.path.join(ROOT, "profiles", "traffic.json")) as fh:
+        with open(os.path.join(ROOT, "profiles", "counters.json")) as fh:
             variant = "normalize" if args.normalize else "fused" if fused else "steps"
-            traffic = json.load(fh).get(args.workload, {}).get(variant, {}).get(dominant)
+            prof = json.load(fh).get(args.workload, {}).get(variant, {})
+            traffic = prof.get("traffic_bytes_per_call", {}).get(dominant)
+            counted_kernel = prof.get("dominant_kernel", {}).get(dominant)
+            counters = prof.get("kernels", {}).get(counted_kernel, {})
     except OSError:
         pass
+    # ceilings of this machine, measured now by the library's probe kernels
+    from gridnet_amd import native
+    ceil = {k: native.probe(k) for k in native.PROBES}
+    lds_peak = LDS_BYTES_PER_CLOCK_PER_CU * CUS * ceil["clock_ghz"]
     dom_s = kernel_s[dominant]
     achieved = bytes_[dominant] / dom_s / 1e9
     # the same entry point against the vector ALU: algorithmic fp32 FMAs per cell-update (27 for
@@ -287,11 +300,31 @@ def main():
             "frac": achieved / HBM_PEAK_GBS,
             "traffic": traffic,
         },
-        # informational: this build compiles with packed fp32 arithmetic switched off, which
-        # halves the vector fp32 peak it can reach
+        # the same entry point against the vector ALU (fp32 FMAs without packed instructions) and
+        # against the LDS pipes; the counter figures are those of the committed profile summary
         "vector_alu": {"kernel": dominant, "achieved": tflops, "unit": "TFLOP/s",
-                       "peak": FP32_PEAK_TFLOPS, "peak_without_packed_fp32": FP32_PEAK_TFLOPS / 2,
-                       "frac": None if tflops is None else tflops / FP32_PEAK_TFLOPS},
+                       "peak": FP32_UNPACKED_PEAK_TFLOPS,
+                       "frac": None if tflops is None else tflops / FP32_UNPACKED_PEAK_TFLOPS,
+                       "measured_fma_ceiling": 2 * ceil["fma_tfma_per_s"],
+                       "frac_of_measured_ceiling": None if tflops is None else tflops / (2 * ceil["fma_tfma_per_s"]),
+                       "valu_busy_pct": counters.get("valu_busy_pct"),
+                       "peak_with_packed_fp32": FP32_PEAK_TFLOPS},
+        "lds": {"kernel": counted_kernel, "unit": "GB/s",
+                "achieved": counters.get("lds_gb_per_s_estimate"),
+                "peak": lds_peak,
+                "frac": None if not counters else counters["lds_gb_per_s_estimate"] / lds_peak,
+                "busy_frac": counters.get("lds_busy_frac"),
+                "bank_conflict_frac_of_busy": counters.get("lds_conflict_frac_of_busy"),
+                "measured_read_ceiling": ceil["lds_gb_per_s"],
+                "peak_is": "128 B per clock and CU x 256 CUs x the measured core clock; 16-byte reads go "
+                           "beyond it on this part, see measured_read_ceiling"},
+        "machine": {"core_clock_ghz_under_load": ceil["clock_ghz"],
+                    "hbm_copy_gb_per_s": ceil["copy_gb_per_s"]},
+        "binds": ("none of HBM, vector ALU and LDS is saturated by the dominant kernel: its waves wait on "
+                  "LDS and ALU latency at 2 waves per SIMD (the register file holds no more of them)")
+                 if wl.block_size == 8 else
+                 ("vector ALU and LDS pipes together (the busier of the two is above 70 % in both step "
+                  "kernels); HBM is far from its limit"),
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(wl)

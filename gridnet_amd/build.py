@@ -11,7 +11,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libgridnet_hip.so")
-SOURCES = ["api.hip", "step_generic.hip", "step_fast.hip", "chain_bwd.hip", "gated_generic.hip", "gated_fast.hip", "layernorm.hip"]
+SOURCES = ["api.hip", "step_generic.hip", "step_fast.hip", "chain_bwd.hip", "gated_generic.hip", "gated_fast.hip", "layernorm.hip", "probe.hip"]
 
 # -packed-fp32-ops is switched OFF on purpose: hipcc -O3 otherwise forms v_pk_*_f32 from
 # ordinary float code.
@@ -47,7 +47,7 @@ def build(verbose: bool = True, extra_flags=(), out=None, objdir=None) -> str:
             print(out)
         return obj
 
-    with ThreadPoolExecutor(max_workers=min(7, len(SOURCES))) as pool:
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
         objs = list(pool.map(compile_one, SOURCES))
     cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", out]
     if verbose:

@@ -1,0 +1,165 @@
+// Machine ceilings measured with the library's own compiler flags, for the benchmark to quote
+// beside the vendor peaks: sustained unpacked fp32 FMA rate, LDS read rate, core clock under load
+// and a plain HBM copy.  Nothing on the update path calls these.
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+
+namespace gridnet {
+namespace {
+
+constexpr int kProbeThreads = 256;
+
+// 16 independent FMA chains per lane, 128 FMAs per trip: enough to hide the ALU latency.
+__global__ __launch_bounds__(kProbeThreads) void probe_fma(float *out, int trips, float a, float b) {
+    float v[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) v[i] = threadIdx.x * 1e-3f + i;
+    for (int t = 0; t < trips; ++t) {
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) v[i] = fmaf(v[i], a, b);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s += v[i];
+    out[(size_t)blockIdx.x * kProbeThreads + threadIdx.x] = s;
+}
+
+// Every lane reads 16 B from consecutive addresses (no bank conflicts), 8 reads per trip.
+__global__ __launch_bounds__(kProbeThreads) void probe_lds(float *out, int trips) {
+    __shared__ __attribute__((aligned(16))) float lds[8192];
+    for (int i = threadIdx.x; i < 8192; i += kProbeThreads) lds[i] = i * 1e-4f;
+    __syncthreads();
+    const float4 *p = reinterpret_cast<const float4 *>(lds);
+    float acc = 0.f;
+    for (int t = 0; t < trips; ++t) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const float4 q = p[(threadIdx.x + 256 * ((u + t) & 7)) & 2047];
+            acc += q.x + q.y + q.z + q.w;
+        }
+    }
+    out[(size_t)blockIdx.x * kProbeThreads + threadIdx.x] = acc;
+}
+
+// Core clock against the fixed 100 MHz counter while every CU runs the FMA loop.
+__global__ __launch_bounds__(kProbeThreads) void probe_clock(float *out, long long *ticks, int trips, float a, float b) {
+    float v[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) v[i] = threadIdx.x * 1e-3f + i;
+    const long long c0 = clock64(), w0 = wall_clock64();
+    for (int t = 0; t < trips; ++t) {
+#pragma unroll
+        for (int r = 0; r < 8; ++r)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) v[i] = fmaf(v[i], a, b);
+    }
+    const long long c1 = clock64(), w1 = wall_clock64();
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) s += v[i];
+    out[(size_t)blockIdx.x * kProbeThreads + threadIdx.x] = s;
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        ticks[0] = c1 - c0;
+        ticks[1] = w1 - w0;
+    }
+}
+
+__global__ __launch_bounds__(kProbeThreads) void probe_copy(const float4 *src, float4 *dst, size_t n) {
+    size_t i = (size_t)blockIdx.x * kProbeThreads + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * kProbeThreads;
+    for (; i < n; i += stride) dst[i] = src[i];
+}
+
+struct Timer {
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    bool ok;
+    Timer() { ok = hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess; }
+    ~Timer() {
+        if (e0) (void)hipEventDestroy(e0);
+        if (e1) (void)hipEventDestroy(e1);
+    }
+    // best of `reps` launches, in seconds; negative on failure
+    template <class F> double best(int reps, F launch) {
+        double best_s = -1.0;
+        for (int r = 0; ok && r < reps; ++r) {
+            if (hipEventRecord(e0, 0) != hipSuccess) return -1.0;
+            launch();
+            if (hipEventRecord(e1, 0) != hipSuccess || hipEventSynchronize(e1) != hipSuccess) return -1.0;
+            float ms = 0.f;
+            if (hipEventElapsedTime(&ms, e0, e1) != hipSuccess) return -1.0;
+            if (best_s < 0 || ms * 1e-3 < best_s) best_s = ms * 1e-3;
+        }
+        return hipGetLastError() == hipSuccess ? best_s : -1.0;
+    }
+};
+
+}  // namespace
+}  // namespace gridnet
+
+using namespace gridnet;
+
+extern "C" int gridnet_hip_probe(int what, double *result) {
+    if (!result) return fail(GRIDNET_ERR_ARGUMENT, "probe: result is null");
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+        return fail(GRIDNET_ERR_LAUNCH, "probe: no device");
+    const int blocks = cus * 8;
+    Timer timer;
+    if (!timer.ok) return fail(GRIDNET_ERR_LAUNCH, "probe: hipEventCreate failed");
+    float *out = nullptr;
+    long long *ticks = nullptr;
+    float4 *src = nullptr, *dst = nullptr;
+    int rc = GRIDNET_OK;
+    double s = -1.0;
+    if (hipMalloc(&out, (size_t)blocks * kProbeThreads * sizeof(float)) != hipSuccess)
+        return fail(GRIDNET_ERR_LAUNCH, "probe: hipMalloc failed");
+    switch (what) {
+    case GRIDNET_PROBE_FMA: {  // TFMA/s (one FMA = 2 flop)
+        const int trips = 4000;
+        s = timer.best(4, [&] { hipLaunchKernelGGL(probe_fma, dim3(blocks), dim3(kProbeThreads), 0, 0, out, trips, 0.999f, 0.001f); });
+        if (s > 0) *result = (double)blocks * kProbeThreads * trips * 128.0 / s / 1e12;
+        break;
+    }
+    case GRIDNET_PROBE_LDS: {  // GB/s over the whole chip
+        const int trips = 4000;
+        s = timer.best(4, [&] { hipLaunchKernelGGL(probe_lds, dim3(blocks), dim3(kProbeThreads), 0, 0, out, trips); });
+        if (s > 0) *result = (double)blocks * kProbeThreads * trips * 8.0 * 16.0 / s / 1e9;
+        break;
+    }
+    case GRIDNET_PROBE_CLOCK: {  // GHz
+        if (hipMalloc(&ticks, 2 * sizeof(long long)) != hipSuccess) { rc = fail(GRIDNET_ERR_LAUNCH, "probe: hipMalloc failed"); break; }
+        const int trips = 4000;
+        s = timer.best(2, [&] { hipLaunchKernelGGL(probe_clock, dim3(blocks), dim3(kProbeThreads), 0, 0, out, ticks, trips, 0.999f, 0.001f); });
+        long long h[2] = {0, 0};
+        if (s > 0 && hipMemcpy(h, ticks, sizeof(h), hipMemcpyDeviceToHost) == hipSuccess && h[1] > 0)
+            *result = (double)h[0] / (double)h[1] * 0.1;
+        else
+            s = -1.0;
+        break;
+    }
+    case GRIDNET_PROBE_COPY: {  // GB/s, read + write
+        const size_t n = (size_t)1 << 26;  // 1 GiB each way
+        if (hipMalloc(&src, n * sizeof(float4)) != hipSuccess || hipMalloc(&dst, n * sizeof(float4)) != hipSuccess) {
+            rc = fail(GRIDNET_ERR_LAUNCH, "probe: hipMalloc failed");
+            break;
+        }
+        hipLaunchKernelGGL(probe_copy, dim3(cus * 16), dim3(kProbeThreads), 0, 0, dst, src, n);  // first touch
+        s = timer.best(4, [&] { hipLaunchKernelGGL(probe_copy, dim3(cus * 16), dim3(kProbeThreads), 0, 0, src, dst, n); });
+        if (s > 0) *result = 2.0 * (double)n * sizeof(float4) / s / 1e9;
+        break;
+    }
+    default:
+        rc = fail(GRIDNET_ERR_ARGUMENT, "probe: unknown quantity");
+    }
+    (void)hipDeviceSynchronize();
+    (void)hipFree(out);
+    if (ticks) (void)hipFree(ticks);
+    if (src) (void)hipFree(src);
+    if (dst) (void)hipFree(dst);
+    if (rc == GRIDNET_OK && s <= 0) rc = fail(GRIDNET_ERR_LAUNCH, "probe: launch or timing failed");
+    return rc;
+}

@@ -46,6 +46,7 @@ EXPORTS = (
     "gridnet_hip_chain_supported",
     "gridnet_hip_chain_halo_floats",
     "gridnet_hip_chain_backward",
+    "gridnet_hip_probe",
 )
 
 
@@ -110,6 +111,8 @@ def _load():
     lib.gridnet_hip_chain_halo_floats.argtypes = [i, i, i, i, i]
     lib.gridnet_hip_chain_backward.restype = i
     lib.gridnet_hip_chain_backward.argtypes = [i] + [p] * 20 + [i] * 8 + [p, z, p]
+    lib.gridnet_hip_probe.restype = i
+    lib.gridnet_hip_probe.argtypes = [i, ctypes.POINTER(ctypes.c_double)]
     return lib
 
 
@@ -117,6 +120,16 @@ try:
     lib = _load()
 except AttributeError as exc:  # an older build of the library without some entry point
     raise ImportError(f"{LIB_PATH} is stale ({exc}): rebuild with `python -m gridnet_amd.build`") from exc
+
+
+PROBES = {"fma_tfma_per_s": 0, "lds_gb_per_s": 1, "clock_ghz": 2, "copy_gb_per_s": 3}  # GRIDNET_PROBE_*
+
+
+def probe(what: str) -> float:
+    """One of the machine ceilings of gridnet_hip_probe on the current device."""
+    out = ctypes.c_double(0.0)
+    check(lib.gridnet_hip_probe(PROBES[what], ctypes.byref(out)))
+    return out.value
 
 
 def last_error() -> str:

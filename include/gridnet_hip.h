@@ -290,6 +290,18 @@ int gridnet_hip_chain_backward(int dtype, const void *weight, const void *bias, 
                                int inner, int block_size, int activation, int flags, void *workspace,
                                size_t workspace_bytes, void *stream);
 
+/*
+ * Machine ceilings, measured with the same compiler flags as the kernels, for a benchmark to
+ * quote beside the vendor's peaks.  No counterpart in the reference and not part of the update
+ * path.  Allocates and frees its own buffers, runs on the null stream and synchronises.
+ *   GRIDNET_PROBE_FMA    sustained fp32 FMA rate without packed instructions, TFMA/s (x2 = TFLOP/s)
+ *   GRIDNET_PROBE_LDS    conflict-free 16-byte LDS reads over all CUs, GB/s
+ *   GRIDNET_PROBE_CLOCK  core clock while every CU runs the FMA loop, GHz
+ *   GRIDNET_PROBE_COPY   device-to-device copy of 1 GiB by a plain kernel, read + write GB/s
+ */
+enum { GRIDNET_PROBE_FMA = 0, GRIDNET_PROBE_LDS = 1, GRIDNET_PROBE_CLOCK = 2, GRIDNET_PROBE_COPY = 3 };
+int gridnet_hip_probe(int what, double *result);
+
 #ifdef __cplusplus
 }
 #endif
