@@ -127,7 +127,7 @@ enum { kTabDst = 0, kTabIn = 2, kTabShellAt = 5, kTabHalo = 6, kTabShellGamma = 
        kTabBeta = 12, kTabGamma = 14, kTabAcc = 16 /* 8 gradient sums */, kTab = 24 };
 constexpr int kChainAffine = 200 * Fetch<ChainTile>::GB;  // packed gamma/beta: 200 half rows
 __host__ __device__ constexpr int chain_lds_floats(int inner) {
-    const int run = 4 * ChainTile::WIN + inner * 512 + kChainAffine + 8 + 9 * 512 + kTab * 256;
+    const int run = 4 * ChainTile::WIN + inner * 512 + kChainAffine + 16 + 9 * 512 + kTab * 256;
     return run > 27 * 512 ? run : 27 * 512;
 }
 __device__ __forceinline__ int stride_of(unsigned code) {
@@ -145,8 +145,8 @@ void chain_bwd(const ChainBwdArgs a) {
     float *dwin = win + 2 * TL::WIN;           // two delta windows, halo zero
     float *hist = dwin + 2 * TL::WIN;          // u_i of this thread's cells at hist + it * 512 + lane * 2
     float *affine = hist + inner * 512;        // gamma and beta of the window, packed per half row
-    float *red = affine + kChainAffine;   // per wave: the two LayerNorm sums of an element
-    float *hwl = red + 8;                      // [256][18]: the weights that feed the shell entries
+    float *red = affine + kChainAffine;   // [2][4][2], per wave: the two LayerNorm sums of an element, elements alternating
+    float *hwl = red + 16;                     // [256][18]: the weights that feed the shell entries
     // ... and what a thread uses once per element: [kTab][256], entry k of thread t at
     // ctab[k * 256 + t].  The register file has no room for these, and a spilled register is
     // worse than an LDS read: spill traffic queues behind the prefetch in the memory pipeline.
@@ -344,32 +344,80 @@ void chain_bwd(const ChainBwdArgs a) {
         if (ln_in) fx.commit_ln(win, pre, affine, nxm, nxr);
         else fx.commit(win, pre);
     };
-    // results are stored one element late, behind the requests of the element after
-    float g_done[CPT], o_done[2];
-    int done_s = -1;
-    auto finish_done = [&]() {
+    // An element is finished one element late.  Its dx is stored behind the requests of the element
+    // after.  With deferred halos, what its delta sums D send to the cells around the block -- the
+    // shell values -- is worked out behind the next element's first barrier, next to the start of
+    // that element's recompute: D waits in a delta window that nothing writes before the sweep, and
+    // the chain of LDS reads, 18 multiply-adds and two wave sums that makes the shell values then
+    // runs beside arithmetic that does not depend on it, instead of holding up every wave of the
+    // workgroup at the end of its own element.
+    float g_done[CPT], o_done[2];     // o_done: the element's D (without deferred halos)
+    float t1_done = 0.f, t2_done = 0.f, nh_done[2] = {0.f, 0.f};  // its LayerNorm sums so far; x-hat at the shell entries
+    int done_s = -1, sums_s = -1;
+    auto store_done = [&]() {
         if (done_s < 0) return;
         const long o = (long)done_s * cells;
         at_bytes<float2>(a.dx + o, ugc) = make_float2(g_done[0], g_done[1]);
-        if (DEFER) {
-            float *rec = a.out2 + (long)done_s * a.nblk * kShell;
+        if (!DEFER) at_bytes<float2>(a.out2 + o, ugc) = make_float2(o_done[0], o_done[1]);
+    };
+    // Where the sources of the thread's two shell entries sit in the D window: read in FRONT of the
+    // barrier, so that the reads behind it start from known addresses (one LDS round trip less).
+    auto shell_sources = [&](unsigned (&hal)[2]) {
+        hal[0] = hal[1] = 0u;
+        if (!DEFER || done_s < 0) return;
+        hal[0] = tab(kTabHalo);
+        hal[1] = tab(kTabHalo + 1);
+    };
+    // behind a barrier that follows the element's last write of D
+    auto shell_of_done = [&](const unsigned (&hals)[2]) {
+        const int hs = done_s;
+        if (DEFER && hs >= 0) {
+            // the thread's 18 shell weights sit side by side (stride 18 floats: nine conflict-free
+            // 64-bit reads)
+            float hwv[18];
 #pragma unroll
-            for (int e = 0; e < 2; ++e)
+            for (int q = 0; q < 9; ++q) {
+                const float2 p2 = *reinterpret_cast<const float2 *>(hwl + tid * 18 + 2 * q);
+                hwv[2 * q] = p2.x;
+                hwv[2 * q + 1] = p2.y;
+            }
+            float t1 = t1_done, t2 = t2_done;
+            float *rec = a.out2 + (long)hs * a.nblk * kShell;
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const unsigned hal = hals[e];
+                const float *src = dwin + TL::WIN + (int)(hal & 0xfffu);
+                // entries 0..255 are the I and J faces: their second stride is 1 (along K), known here,
+                // so that the three reads of a row get constant offsets from one address
+                const int sb = stride_of((hal >> 12) & 3u), sc = e == 0 ? 1 : stride_of((hal >> 14) & 3u);
+                float acc = 0.f;
+#pragma unroll
+                for (int slot = 0; slot < 9; ++slot)
+                    acc = fmaf(hwv[e * 9 + slot], src[(slot / 3 - 1) * sb + (slot % 3 - 1) * sc], acc);
+                t1 = fmaf(__uint_as_float(tab(kTabShellGamma + e)), acc, t1);
+                t2 = fmaf(acc, nh_done[e] - __uint_as_float(tab(kTabShellBeta + e)), t2);
                 if (s_in[e]) {
                     // opaque here, so that the offset is widened inside this block, where the
                     // store can still take it as a 32-bit lane offset beside the scalar base
                     unsigned off = tab(kTabDst + e);
                     asm volatile("" : "+v"(off));
-                    at_bytes<float>(rec, off) = o_done[e];
+                    at_bytes<float>(rec, off) = acc;
                 }
-            if (tid == 0) {  // the four waves' sums, in a fixed order
-                float *to = a.x_part + ((long)done_s * a.nblk + blk) * 2;
-                to[0] = (red[0] + red[2]) + (red[4] + red[6]);
-                to[1] = (red[1] + red[3]) + (red[5] + red[7]);
             }
-        } else {
-            at_bytes<float2>(a.out2 + o, ugc) = make_float2(o_done[0], o_done[1]);
+            t1 = slot_wave_sum<256>(t1);
+            t2 = slot_wave_sum<256>(t2);
+            if ((tid & 63) == 0)
+                *reinterpret_cast<float2 *>(red + (hs & 1) * 8 + 2 * (tid >> 6)) = make_float2(t1, t2);
         }
+        // the sums of the element before that one: its four waves' shares, in a fixed order (they
+        // were written a barrier ago, into the other half of `red`)
+        if (DEFER && sums_s >= 0 && tid == 0) {
+            const float *r = red + (sums_s & 1) * 8;
+            float *to = a.x_part + ((long)sums_s * a.nblk + blk) * 2;
+            to[0] = (r[0] + r[2]) + (r[4] + r[6]);
+            to[1] = (r[1] + r[3]) + (r[5] + r[7]);
+        }
+        sums_s = hs;
         done_s = -1;
     };
 
@@ -380,10 +428,11 @@ void chain_bwd(const ChainBwdArgs a) {
     }
     for (int s = s0; s < s1; ++s) {
         take_turns(s);
-        lds_barrier();  // this element's window is in place; the last round's LDS readers are done
         // Requests first, stores behind them: loads and stores retire through one in-order
         // counter, and no wait for a load may include the stores.  This element's gradient (used
-        // after the recompute, which hides the trip), then the next element's window.
+        // after the recompute, which hides the trip), then the next element's window.  All of it
+        // in front of the barrier: none of it touches the windows, and the wait for the other
+        // waves covers the issue.
         const long at = (long)s * cells;
         const float2 dy2 = at_bytes<float2>(a.dy + at, ugc), yr2 = at_bytes<float2>(a.y_raw + at, ugc);
         const float *rec = hin + ((long)s * a.nblk + blk) * kShell;
@@ -396,7 +445,11 @@ void chain_bwd(const ChainBwdArgs a) {
         const float ny0 = load_ahead(a.y_stats, 2 * s), ny1 = load_ahead(a.y_stats, 2 * s + 1),
                     ny2 = load_ahead(a.y_sums, 2 * s), ny3 = load_ahead(a.y_sums, 2 * s + 1);
         fetch_window(min(s + 1, s1 - 1));
-        finish_done();
+        store_done();
+        unsigned shc[2];
+        shell_sources(shc);
+        lds_barrier();  // this element's window is in place; the last round's LDS readers are done
+        shell_of_done(shc);
 
         // ---- forward recompute; u_i of the owned cells is remembered ----
         float xcur[CPT];
@@ -496,59 +549,34 @@ void chain_bwd(const ChainBwdArgs a) {
             acc_ref(2 + c) += dre[c];
         }
 
-        float out[2];
         if (DEFER) {
-            // D into the delta window that the last gather did not read (its halo is zero)
+            // D into the delta window that the last gather did not read (its halo is zero); the own
+            // cells' share of the two LayerNorm sums
 #pragma unroll
             for (int c = 0; c < CPT; ++c) dwin[TL::WIN + pl.own + c] = dsum[c];
-
             const float bet0 = __uint_as_float(tab(kTabBeta)), bet1 = __uint_as_float(tab(kTabBeta + 1));
-            float t1 = fmaf(__uint_as_float(tab(kTabGamma)), g[0], __uint_as_float(tab(kTabGamma + 1)) * g[1]);
-            float t2 = fmaf(g[0], xcur[0] - bet0, g[1] * (xcur[1] - bet1));
-            lds_barrier();
-            // the thread's 18 shell weights sit side by side (stride 18 floats: nine conflict-free
-            // 64-bit reads)
-            float hwv[18];
-#pragma unroll
-            for (int k = 0; k < 9; ++k) {
-                const float2 p2 = *reinterpret_cast<const float2 *>(hwl + tid * 18 + 2 * k);
-                hwv[2 * k] = p2.x;
-                hwv[2 * k + 1] = p2.y;
-            }
-#pragma unroll
-            for (int e = 0; e < 2; ++e) {
-                const unsigned hal = tab(kTabHalo + e);
-                const float *src = dwin + TL::WIN + (int)(hal & 0xfffu);
-                // entries 0..255 are the I and J faces: their second stride is 1 (along K), known here,
-                // so that the three reads of a row get constant offsets from one address
-                const int sb = stride_of((hal >> 12) & 3u), sc = e == 0 ? 1 : stride_of((hal >> 14) & 3u);
-                float acc = 0.f;
-#pragma unroll
-                for (int slot = 0; slot < 9; ++slot)
-                    acc = fmaf(hwv[e * 9 + slot], src[(slot / 3 - 1) * sb + (slot % 3 - 1) * sc], acc);
-                out[e] = acc;
-                t1 = fmaf(__uint_as_float(tab(kTabShellGamma + e)), acc, t1);
-                t2 = fmaf(acc, nh[e] - __uint_as_float(tab(kTabShellBeta + e)), t2);
-            }
-            t1 = slot_wave_sum<256>(t1);
-            t2 = slot_wave_sum<256>(t2);
-            if ((tid & 63) == 0) *reinterpret_cast<float2 *>(red + 2 * (tid >> 6)) = make_float2(t1, t2);
+            t1_done = fmaf(__uint_as_float(tab(kTabGamma)), g[0], __uint_as_float(tab(kTabGamma + 1)) * g[1]);
+            t2_done = fmaf(g[0], xcur[0] - bet0, g[1] * (xcur[1] - bet1));
+            nh_done[0] = nh[0];
+            nh_done[1] = nh[1];
         } else {
             if (inner == 0) lds_barrier();
 #pragma unroll
-            for (int c = 0; c < CPT; ++c) out[c] = dsum[c];
+            for (int c = 0; c < CPT; ++c) o_done[c] = dsum[c];
         }
         done_s = s;
 #pragma unroll
-        for (int c = 0; c < CPT; ++c) {
-            g_done[c] = g[c];
-            o_done[c] = out[c];
-        }
+        for (int c = 0; c < CPT; ++c) g_done[c] = g[c];
         // the x windows are free (nothing reads them after the last barrier of the sweep)
         if (s + 1 < s1) commit_window();
     }
-    lds_barrier();  // the last element's sums
-    finish_done();
+    store_done();
+    unsigned shc[2];
+    shell_sources(shc);
+    lds_barrier();  // the last element's D
+    shell_of_done(shc);
+    lds_barrier();  // its sums
+    shell_of_done(shc);
 
     // ---- parameter gradients ----
 #pragma unroll
