@@ -34,8 +34,13 @@ template <typename T> __device__ __forceinline__ T sigmoid_stable(T u) {
 
 template <int ACT, typename T> struct Act;
 
+// max as one instruction (a compare and a select otherwise); max(u, 0) and, for a slope below
+// one, max(u, slope * u) are relu and leaky_relu for every u, signed zeros and NaN included
+__device__ __forceinline__ float max_of(float a, float b) { return __builtin_fmaxf(a, b); }
+__device__ __forceinline__ double max_of(double a, double b) { return __builtin_fmax(a, b); }
+
 template <typename T> struct Act<GRIDNET_ACT_RELU, T> {
-    static __device__ __forceinline__ T f(T u) { return u > T(0) ? u : T(0); }
+    static __device__ __forceinline__ T f(T u) { return max_of(u, T(0)); }
     static __device__ __forceinline__ void fd(T u, T &f, T &d) {
         bool pos = u > T(0);
         f = pos ? u : T(0);
@@ -43,7 +48,7 @@ template <typename T> struct Act<GRIDNET_ACT_RELU, T> {
     }
 };
 template <typename T> struct Act<GRIDNET_ACT_LEAKY_RELU, T> {
-    static __device__ __forceinline__ T f(T u) { return u > T(0) ? u : T(0.01) * u; }
+    static __device__ __forceinline__ T f(T u) { return max_of(u, T(0.01) * u); }
     static __device__ __forceinline__ void fd(T u, T &f, T &d) {
         bool pos = u > T(0);
         f = pos ? u : T(0.01) * u;
