@@ -54,13 +54,18 @@ template <int TPS> __device__ __forceinline__ void slot_barrier() {
     }
 }
 
-// The workgroups that share a CU take turns at the higher wave priority, two batch elements at
-// a time.  Left alone the arbiter keeps preferring the waves of the older workgroup, which then
-// finishes early and leaves the CU half empty for the rest of the kernel (workgroups of the
-// forward kernel ended anywhere between 46 and 68 us after the start); which workgroups share a
-// CU is not known, so the turn is derived from the workgroup id, and a pair that happens to get
-// the same turns loses nothing.  Measured: 2-3 % on the forward and the first backward kernel
-// with 8^3 blocks (nothing, or a loss, in the forward kernel for 4^3 blocks, which does without).
+// Wave priority as a function of the element a workgroup is working on: high for two elements, low
+// for the next two.  Left alone the arbiter keeps preferring the waves of the older workgroup of a
+// CU, which then finishes early and leaves the CU half empty for the rest of the kernel (workgroups
+// of the forward kernel ended anywhere between 46 and 68 us after the start).  With this schedule
+// two workgroups that work on the same element have equal priority, and when one falls behind it
+// is the one with the higher priority for part of the time: their progress stays within two
+// elements.  What matters is that workgroups sharing a CU follow the SAME schedule: measured on the
+// chain's backward kernel (one round of 512 workgroups, 64^3 grid, batch 32), any of the block id's
+// low bits as phase gives 203 us, no priorities 215 us, and a phase taken from bit 8 of the block id
+// -- opposite schedules for the two workgroups of a CU, which the dispatcher places 256 ids apart --
+// 214 us; periods of 1, 4 and 8 elements give 206, 209 and 211 us.  2-3 % on the forward kernel with
+// 8^3 blocks (nothing, or a loss, in the forward kernel for 4^3 blocks, which does without).
 __device__ __forceinline__ void take_turns(int element) {
     if (((element >> 1) ^ blockIdx.x ^ (blockIdx.x >> 2)) & 1) __builtin_amdgcn_s_setprio(1);
     else __builtin_amdgcn_s_setprio(0);
