@@ -129,14 +129,28 @@ int gridnet_hip_forward(int dtype, const void *weight, const void *bias, const v
     return step_forward_generic(a, st);
 }
 
+// What lies behind the first `used` bytes of a workspace (rounded up to 256) is room for the
+// gradient copies of a split batch (launch.h: StepArgs::slabs); callers that hand over only the
+// required part get a batch that is split less, the result is the same.
+static void give_slabs(StepArgs &a, void *workspace, size_t workspace_bytes, size_t used) {
+    const size_t at = (used + 255) / 256 * 256;
+    a.slabs = nullptr;
+    a.slab_bytes = 0;
+    if (workspace && workspace_bytes > at) {
+        a.slabs = (char *)workspace + at;
+        a.slab_bytes = workspace_bytes - at;
+    }
+}
+
 size_t gridnet_hip_backward_workspace_bytes(int dtype, int B, int M, int N, int K, int inner,
                                             int block_size, int normalize) {
     StepArgs a{};
     a.dtype = dtype; a.B = B; a.M = M; a.N = N; a.K = K; a.inner = inner;
     a.block_size = block_size; a.normalize = normalize != 0; a.activation = GRIDNET_ACT_RELU;
     if (B <= 0 || M <= 0 || N <= 0 || K <= 0) return 0;
-    if (step_fast_supports(a, true)) return step_fast_backward_workspace(a);
-    return 0;
+    if (!step_fast_supports(a, true)) return 0;
+    const size_t slabs = step_fast_slab_bytes(a);
+    return slabs ? (step_fast_backward_workspace(a) + 255) / 256 * 256 + slabs : step_fast_backward_workspace(a);
 }
 
 static int backward_step(int dtype, const void *weight, const void *bias, const void *scale,
@@ -168,6 +182,7 @@ static int backward_step(int dtype, const void *weight, const void *bias, const 
         return fail(GRIDNET_ERR_WORKSPACE, "backward needs %zu bytes of workspace, got %zu", need,
                     workspace ? workspace_bytes : (size_t)0);
     a.workspace = workspace; a.workspace_bytes = workspace_bytes;
+    give_slabs(a, workspace, workspace_bytes, need);
     return step_backward_fast(a, st);
 }
 
@@ -217,8 +232,9 @@ size_t gridnet_hip_backward_gated_workspace_bytes(int dtype, int B, int M, int N
     a.dtype = dtype; a.B = B; a.M = M; a.N = N; a.K = K; a.inner = inner;
     a.block_size = block_size; a.activation = GRIDNET_ACT_RELU;
     if (B <= 0 || M <= 0 || N <= 0 || K <= 0) return 0;
-    if (gated_fast_supports(a, true)) return gated_fast_backward_workspace(a);
-    return 0;
+    if (!gated_fast_supports(a, true)) return 0;
+    const size_t slabs = gated_fast_slab_bytes(a);
+    return slabs ? (gated_fast_backward_workspace(a) + 255) / 256 * 256 + slabs : gated_fast_backward_workspace(a);
 }
 
 int gridnet_hip_backward_gated(int dtype, const void *weight, const void *bias, const void *x,
@@ -240,6 +256,7 @@ int gridnet_hip_backward_gated(int dtype, const void *weight, const void *bias, 
         if (!workspace || workspace_bytes < need)
             return fail(GRIDNET_ERR_WORKSPACE, "backward needs %zu bytes of workspace, got %zu", need,
                         workspace ? workspace_bytes : (size_t)0);
+        give_slabs(a, workspace, workspace_bytes, need);
         return gated_backward_fast(a, (hipStream_t)stream);
     }
     return gated_backward(a, (hipStream_t)stream);
@@ -326,7 +343,8 @@ size_t gridnet_hip_fused_workspace_bytes(int B, int M, int N, int K, int inner, 
     a.block_size = block_size; a.activation = GRIDNET_ACT_RELU;
     if (B <= 0 || M <= 0 || N <= 0 || K <= 0 || (block_size != 4 && block_size != 8)) return 0;
     if (!backward) return fused_forward_workspace(a);
-    return fused_backward_dsum(a) + fused_backward_parts(a);
+    const size_t need = fused_backward_dsum(a) + fused_backward_parts(a), slabs = step_fast_slab_bytes(a);
+    return slabs ? (need + 255) / 256 * 256 + slabs : need;
 }
 
 static int fused_forward(int dtype, const void *weight, const void *bias, const void *scale,
@@ -444,6 +462,7 @@ static int fused_backward(int dtype, const void *weight, const void *bias, const
                     workspace ? workspace_bytes : (size_t)0);
     hipStream_t st = (hipStream_t)stream;
     a.workspace = workspace; a.workspace_bytes = dsum_bytes;
+    give_slabs(a, workspace, workspace_bytes, need);
     a.ln.beta = (const float *)beta;
     a.ln.x_stats = (const float *)x_stats;
     a.ln.y_raw = (const float *)y_raw;
@@ -540,6 +559,7 @@ int gridnet_hip_chain_backward(int dtype, const void *weight, const void *bias, 
                     workspace ? workspace_bytes : (size_t)0);
     hipStream_t st = (hipStream_t)stream;
     a.workspace = workspace; a.workspace_bytes = dsum_bytes;
+    give_slabs(a, workspace, workspace_bytes, need);
     a.ln.beta = (const float *)beta;
     a.ln.x_stats = (const float *)x_stats;
     a.ln.y_raw = (const float *)y_raw;

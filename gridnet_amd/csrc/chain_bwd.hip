@@ -111,6 +111,7 @@ struct ChainBwdArgs {
     float *out2;               // DEFER: halo_out [B, nblk, 488]; otherwise D [B, cells]
     float *x_part;             // DEFER: [B, nblk, 2] sums for the LayerNorm in front of this step
     int B, M, N, K, inner, nblk, nchunk, chunk_len, param_mode;
+    long slab_stride;          // split batch: floats between the chunks' copies of the gradient arrays, else 0
 };
 
 // LDS (floats): [x window x2 | delta window x2 | u_i of the owned cells, inner slabs of 512 |
@@ -154,6 +155,13 @@ void chain_bwd(const ChainBwdArgs a) {
 
     int blk, chunk;
     if (!split_block_id(blockIdx.x, a.nblk, a.nchunk, blk, chunk)) return;  // grid padding
+    // A split batch: every chunk commits into a copy of the gradient arrays of its own.  Worked out
+    // where it is used (before and after the batch loop), not kept: the loop has no register to spare.
+    auto slab_offset = [&]() -> long {
+        int b2, c2;
+        (void)split_block_id(blockIdx.x, a.nblk, a.nchunk, b2, c2);
+        return a.slab_stride ? c2 * a.slab_stride : 0;
+    };
     const int tid = threadIdx.x;
     const Place<TL, CPT, 1> pl(tid, blk, a.N, a.K);
     const Fetch<TL> fx(tid, pl.p0, pl.q0, pl.r0, a.M, a.N, a.K);
@@ -313,16 +321,17 @@ void chain_bwd(const ChainBwdArgs a) {
     for (int idx = tid; idx < 2 * TL::WIN; idx += 256) dwin[idx] = 0.f;
     wait_global_loads();
     if (a.param_mode == kParamAddExclusive) {
+        const long slab_off = slab_offset();
         // the accumulators start from what the gradient buffers hold and are stored at the end;
         // requested here, behind the set-up wait, the old values arrive during the first element
 #pragma unroll
         for (int t = 0; t < 27; ++t)
 #pragma unroll
-            for (int c = 0; c < CPT; ++c) nw[t][c] = a.dweight[owner_of(t, c)];
-        load_cells<CPT>(a.dbias + pl.gc, db);
-        load_cells<CPT>(a.dscale + pl.gc, dr);
-        load_cells<CPT>(a.dgamma + pl.gc, dgam);
-        load_cells<CPT>(a.dbeta + pl.gc, dbet);
+            for (int c = 0; c < CPT; ++c) nw[t][c] = (a.dweight + slab_off)[owner_of(t, c)];
+        load_cells<CPT>((a.dbias + slab_off) + pl.gc, db);
+        load_cells<CPT>((a.dscale + slab_off) + pl.gc, dr);
+        load_cells<CPT>((a.dgamma + slab_off) + pl.gc, dgam);
+        load_cells<CPT>((a.dbeta + slab_off) + pl.gc, dbet);
     }
     auto acc_ref = [&](int k) -> float & { return reinterpret_cast<float *>(ctab)[(kTabAcc + k) * 256 + tid]; };
 #pragma unroll
@@ -579,6 +588,7 @@ void chain_bwd(const ChainBwdArgs a) {
     shell_of_done(shc);
 
     // ---- parameter gradients ----
+    const long slab_off = slab_offset();
 #pragma unroll
     for (int c = 0; c < CPT; ++c) {
         db[c] = acc_ref(c);
@@ -586,21 +596,21 @@ void chain_bwd(const ChainBwdArgs a) {
         dgam[c] = acc_ref(4 + c);
         dbet[c] = acc_ref(6 + c);
     }
-    commit_grads<27, CPT>(a.dweight, nw, a.param_mode, owner_of, always);
+    commit_grads<27, CPT>((a.dweight + slab_off), nw, a.param_mode, owner_of, always);
     float one[1][CPT];
     auto own_cell = [&](int, int c) { return pl.gc + c; };
 #pragma unroll
     for (int c = 0; c < CPT; ++c) one[0][c] = db[c];
-    commit_grads<1, CPT>(a.dbias, one, a.param_mode, own_cell, always);
+    commit_grads<1, CPT>((a.dbias + slab_off), one, a.param_mode, own_cell, always);
 #pragma unroll
     for (int c = 0; c < CPT; ++c) one[0][c] = dr[c];
-    commit_grads<1, CPT>(a.dscale, one, a.param_mode, own_cell, always);
+    commit_grads<1, CPT>((a.dscale + slab_off), one, a.param_mode, own_cell, always);
 #pragma unroll
     for (int c = 0; c < CPT; ++c) one[0][c] = dgam[c];
-    commit_grads<1, CPT>(a.dgamma, one, a.param_mode, own_cell, always);
+    commit_grads<1, CPT>((a.dgamma + slab_off), one, a.param_mode, own_cell, always);
 #pragma unroll
     for (int c = 0; c < CPT; ++c) one[0][c] = dbet[c];
-    commit_grads<1, CPT>(a.dbeta, one, a.param_mode, own_cell, always);
+    commit_grads<1, CPT>((a.dbeta + slab_off), one, a.param_mode, own_cell, always);
 }
 
 template <int ACT, bool DEFER> int launch_chain(const StepArgs &a, hipStream_t st) {
@@ -629,29 +639,44 @@ template <int ACT, bool DEFER> int launch_chain(const StepArgs &a, hipStream_t s
     const bool whole = k.nblk >= plan_device_cus();
     plan_batch_chunks(a.B, k.nblk, 1, per_cu * plan_device_cus(), whole, k.nchunk, k.chunk_len);
     const bool new_params = (a.flags & GRIDNET_OVERWRITE_PARAMS) != 0;
-    k.param_mode = kParamAtomic;
-    if (k.nchunk == 1) {
-        k.param_mode = new_params ? kParamStore : kParamAddExclusive;
-    } else if (new_params) {
-        if (int rc = plan_fill_zero((float *)a.dweight, 27 * cells, st)) return rc;
-        if (int rc = plan_fill_zero((float *)a.dbias, cells, st)) return rc;
-        if (int rc = plan_fill_zero((float *)a.dscale, cells, st)) return rc;
-        if (int rc = plan_fill_zero(a.ln.dgamma, cells, st)) return rc;
-        if (int rc = plan_fill_zero(a.ln.dbeta, cells, st)) return rc;
+    // A split batch: every chunk gets a copy of the gradient arrays in the scratch; with less
+    // room than chunks the batch is split less (down to not at all).
+    const long slab_floats = kStepSlabPlanes * cells;
+    if (k.nchunk > 1) {
+        const int room = plan_slab_capacity(a.slabs, a.slab_bytes, slab_floats);
+        if (room < k.nchunk)
+            plan_batch_chunks(a.B, k.nblk, 1, (room < 2 ? 1 : room) * k.nblk, room < 2, k.nchunk, k.chunk_len);
     }
+    const bool split = k.nchunk > 1;
+    k.param_mode = split || new_params ? kParamStore : kParamAddExclusive;
+    k.slab_stride = split ? slab_floats : 0;
+    float *slab = (float *)a.slabs;
     k.weight = (const float *)a.weight; k.bias = (const float *)a.bias; k.scale = (const float *)a.scale;
     k.gamma = a.ln.gamma; k.beta = a.ln.beta;
     k.x = (const float *)a.x; k.x_stats = a.ln.x_stats;
     k.dy = (const float *)a.dy; k.y_raw = a.ln.y_raw; k.y_stats = a.ln.y_stats; k.y_sums = a.ln.y_sums;
     k.halo_in = a.ln.halo_in;
-    k.dweight = (float *)a.dweight; k.dbias = (float *)a.dbias; k.dscale = (float *)a.dscale;
-    k.dgamma = a.ln.dgamma; k.dbeta = a.ln.dbeta;
+    k.dweight = split ? slab : (float *)a.dweight;
+    k.dbias = split ? slab + 27 * cells : (float *)a.dbias;
+    k.dscale = split ? slab + 28 * cells : (float *)a.dscale;
+    k.dgamma = split ? slab + 29 * cells : a.ln.dgamma;
+    k.dbeta = split ? slab + 30 * cells : a.ln.dbeta;
     k.dx = (float *)a.dx;
     k.out2 = DEFER ? a.ln.halo_out : (float *)a.workspace;
     k.x_part = a.ln.x_part;
     k.B = a.B; k.M = a.M; k.N = a.N; k.K = a.K; k.inner = a.inner;
     hipLaunchKernelGGL(kern, dim3(padded_grid(k.nblk, k.nchunk)), dim3(256), lds, st, k);
     if (int rc = check_launch("chain_bwd")) return rc;
+    if (split) {
+        SlabTargets t{};
+        t.dst[0] = (float *)a.dweight; t.end[0] = 27 * cells;
+        t.dst[1] = (float *)a.dbias;   t.end[1] = 28 * cells;
+        t.dst[2] = (float *)a.dscale;  t.end[2] = 29 * cells;
+        t.dst[3] = a.ln.dgamma;        t.end[3] = 30 * cells;
+        t.dst[4] = a.ln.dbeta;         t.end[4] = 31 * cells;
+        t.count = 5;
+        if (int rc = plan_reduce_slabs(slab, k.nchunk, slab_floats, t, new_params ? 0 : 1, st)) return rc;
+    }
     if (DEFER) return GRIDNET_OK;
     // dx is wanted finished: the cross-block kernel completes it from D (same blocks, same chunks)
     return step_cross_launch(a, k.nchunk, k.chunk_len, st);

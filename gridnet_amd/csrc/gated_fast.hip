@@ -17,6 +17,7 @@
 
 #include "common.h"
 #include "fast_tiles.h"
+#include "plan.h"
 #include "launch.h"
 
 namespace gridnet {
@@ -132,13 +133,17 @@ void gated_bwd_fast(const float *__restrict__ weight, const float *__restrict__ 
                     const float *__restrict__ x, const float *__restrict__ dy,
                     float *__restrict__ dweight, float *__restrict__ dbias, float *__restrict__ dx,
                     float *__restrict__ dsum_out, int B, int M, int N, int K, int inner, int nblk,
-                    int nchunk, int chunk_len, int param_mode, int dx_accumulate) {
+                    int nchunk, int chunk_len, int param_mode, int dx_accumulate, long slab_stride) {
     using TL = Tile<BS, 1>;
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int slot_floats = gated_slot_floats<BS>(inner);
 
     int blk, chunk;
     if (!split_block_id(blockIdx.x, nblk, nchunk, blk, chunk)) return;  // grid padding
+    if (slab_stride) {  // a split batch: every chunk commits into a copy of the gradient arrays of its own
+        dweight += chunk * slab_stride;
+        dbias += chunk * slab_stride;
+    }
     const Place<TL, 1, NSLOT> pl(threadIdx.x, blk, N, K);
     const Fetch<TL> fx(pl.lane, pl.p0, pl.q0, pl.r0, M, N, K);
     float *win = lds + pl.slot * slot_floats;
@@ -362,23 +367,16 @@ void gated_bwd_fast(const float *__restrict__ weight, const float *__restrict__ 
         reduce(dbg);
         if (pl.slot != 0) return;
     }
-    if (param_mode != kParamAtomic) {
+    // plain stores in every mode: this workgroup is the only one that writes these entries of its
+    // arrays (the caller's, or its chunk's copy of them), and the accumulating mode started from
+    // the old contents
 #pragma unroll
-        for (int t = 0; t < 27; ++t) {
-            dweight[owner_of(t, 0)] = na[t];
-            dweight[owner_of(t, 1)] = ng[t];
-        }
-        dbias[pl.gc] = dba;
-        dbias[cells + pl.gc] = dbg;
-    } else {
-#pragma unroll
-        for (int t = 0; t < 27; ++t) {
-            unsafeAtomicAdd(dweight + owner_of(t, 0), na[t]);
-            unsafeAtomicAdd(dweight + owner_of(t, 1), ng[t]);
-        }
-        unsafeAtomicAdd(dbias + pl.gc, dba);
-        unsafeAtomicAdd(dbias + cells + pl.gc, dbg);
+    for (int t = 0; t < 27; ++t) {
+        dweight[owner_of(t, 0)] = na[t];
+        dweight[owner_of(t, 1)] = ng[t];
     }
+    dbias[pl.gc] = dba;
+    dbias[cells + pl.gc] = dbg;
 }
 
 __global__ void gated_fast_fill_zero(float *p, long n) {
@@ -472,20 +470,31 @@ template <int BS, int NSLOT, int ACT> int launch_bwd(const StepArgs &a, hipStrea
     int nchunk, chunk_len;
     plan_chunks(a.B, nblk, NSLOT, per_cu * device_cus(), nblk >= device_cus(), nchunk, chunk_len);
     const bool new_params = (a.flags & GRIDNET_OVERWRITE_PARAMS) != 0;
-    int param_mode = kParamAtomic;
-    if (nchunk == 1) {
-        param_mode = new_params ? kParamStore : kParamAddExclusive;
-    } else if (new_params) {
-        if (int rc = fill_zero((float *)a.dweight, 54 * cells, st)) return rc;
-        if (int rc = fill_zero((float *)a.dbias, 2 * cells, st)) return rc;
+    // A split batch: every chunk gets a copy of the gradient arrays in the scratch; with less
+    // room than chunks the batch is split less (down to not at all).
+    const long slab_floats = kGatedSlabPlanes * cells;
+    if (nchunk > 1) {
+        const int room = plan_slab_capacity(a.slabs, a.slab_bytes, slab_floats);
+        if (room < nchunk) plan_chunks(a.B, nblk, NSLOT, (room < 2 ? 1 : room) * nblk, room < 2, nchunk, chunk_len);
     }
+    const bool split = nchunk > 1;
+    const int param_mode = split || new_params ? kParamStore : kParamAddExclusive;
+    float *slab = (float *)a.slabs;
     const int dx_accumulate = (a.flags & GRIDNET_OVERWRITE_DX) ? 0 : 1;
     hipLaunchKernelGGL(kern, dim3(padded_grid(nblk, nchunk)), dim3(TL::TPS * NSLOT), lds, st,
                        (const float *)a.weight, (const float *)a.bias, (const float *)a.x,
-                       (const float *)a.dy, (float *)a.dweight, (float *)a.dbias, (float *)a.dx,
+                       (const float *)a.dy, split ? slab : (float *)a.dweight,
+                       split ? slab + 54 * cells : (float *)a.dbias, (float *)a.dx,
                        (float *)a.workspace, a.B, a.M, a.N, a.K, a.inner, nblk, nchunk, chunk_len,
-                       param_mode, dx_accumulate);
+                       param_mode, dx_accumulate, split ? slab_floats : 0L);
     if (int rc = check_launch("gated_bwd_fast")) return rc;
+    if (split) {
+        SlabTargets t{};
+        t.dst[0] = (float *)a.dweight; t.end[0] = 54 * cells;
+        t.dst[1] = (float *)a.dbias;   t.end[1] = 56 * cells;
+        t.count = 2;
+        if (int rc = plan_reduce_slabs(slab, nchunk, slab_floats, t, new_params ? 0 : 1, st)) return rc;
+    }
     // same blocks, same batch chunks; the parameter gradients are complete, dx is not yet
     return gated_cross_launch(a, (const float *)a.workspace, nchunk, chunk_len, st);
 }
@@ -521,6 +530,18 @@ bool gated_fast_supports(const StepArgs &a, bool backward) {
 size_t gated_fast_backward_workspace(const StepArgs &a) {
     // D0 and D1 of every cell, handed from gated_bwd_fast to the cross-block kernel
     return (size_t)2 * a.B * a.M * a.N * a.K * sizeof(float);
+}
+
+size_t gated_fast_slab_bytes(const StepArgs &a) {
+    // the most chunks any plan of the backward kernel makes (see step_fast_slab_bytes)
+    const long nblk = (long)(a.M / a.block_size) * (a.N / a.block_size) * (a.K / a.block_size);
+    if (nblk >= device_cus()) return 0;
+    const int nslot = a.block_size == 8 ? kBwdSlots8 : kBwdSlots4;
+    long chunks = (long)(a.block_size == 8 ? 2 : 16) * device_cus() / nblk;
+    const long most = (a.B + nslot - 1) / nslot;
+    if (chunks > most) chunks = most;
+    if (chunks < 2) return 0;
+    return (size_t)chunks * kGatedSlabPlanes * a.M * a.N * a.K * sizeof(float);
 }
 
 int gated_forward_fast(const StepArgs &a, hipStream_t st) { return dispatch<false>(a, st); }

@@ -57,13 +57,23 @@ struct StepArgs {
     void *workspace;
     size_t workspace_bytes;
     LnFold ln;  // all null: the plain step
+    // backward on grids where the batch of a block is split over workgroups: room for every
+    // chunk's own copy of the gradient arrays (see plan.h); may be null (the batch is then not split)
+    void *slabs;
+    size_t slab_bytes;
 };
+
+// floats per cell in one copy of the plain step's gradient arrays (see plan.h): 27 weight planes,
+// bias, scale and, with the folded LayerNorm, gamma and beta
+constexpr int kStepSlabPlanes = 31;
+// ... and of the gated step's: 54 weight planes, 2 bias planes
+constexpr int kGatedSlabPlanes = 56;
 
 // How a workgroup commits its parameter gradients.
 enum ParamMode {
     kParamStore = 0,         // sole owner of the cells, output uninitialised: plain store
     kParamAddExclusive = 1,  // sole owner, output holds a prior sum: read-add-write
-    kParamAtomic = 2         // several workgroups (batch chunks) share the cells
+    kParamAtomic = 2         // several workgroups (batch chunks) share the cells (generic kernels only)
 };
 
 struct LayerNormArgs {
@@ -84,7 +94,8 @@ int step_backward_generic(const StepArgs &a, hipStream_t st);
 
 // step_fast.hip: fp32, block sizes 4 and 8, normalize on or off (off only with the folded LayerNorm)
 bool step_fast_supports(const StepArgs &a, bool backward);
-size_t step_fast_backward_workspace(const StepArgs &a);
+size_t step_fast_backward_workspace(const StepArgs &a);   // what the backward cannot do without
+size_t step_fast_slab_bytes(const StepArgs &a);           // room for the gradient copies of a split batch
 int step_forward_fast(const StepArgs &a, hipStream_t st);
 int step_backward_fast(const StepArgs &a, hipStream_t st);
 // partial statistics per (block, batch element) that the kernels above write when asked to
@@ -108,6 +119,7 @@ int gated_cross_launch(const StepArgs &a, const float *dsum, int nchunk, int chu
 // gated_fast.hip: fp32, block sizes 4 and 8, as many inner iterations as the LDS holds
 bool gated_fast_supports(const StepArgs &a, bool backward);
 size_t gated_fast_backward_workspace(const StepArgs &a);
+size_t gated_fast_slab_bytes(const StepArgs &a);
 int gated_forward_fast(const StepArgs &a, hipStream_t st);
 int gated_backward_fast(const StepArgs &a, hipStream_t st);
 

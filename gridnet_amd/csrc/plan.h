@@ -50,6 +50,58 @@ int plan_fill_zero(float *p, long n, hipStream_t st) {
     return check_launch("fill_zero");
 }
 
+// ---- parameter gradients of a batch that is split over workgroups -----------------------------
+// On grids with fewer blocks than the chip has CUs the batch of a block is dealt to several
+// workgroups.  Each of them leaves its share of the gradient arrays in a copy of its own (a
+// "slab": the arrays one behind the other, `planes` x cells floats) with plain stores, and one
+// small kernel adds the copies in chunk order into the caller's arrays: no atomics, the same bits
+// on every run.
+struct SlabTargets {
+    float *dst[5];   // the caller's gradient arrays, in slab order
+    long end[5];     // end of each array within a slab, in floats (multiples of 4)
+    int count;
+};
+
+__global__ void plan_reduce_slabs_f32(const float *slabs, int ncopies, long stride, SlabTargets t,
+                                      long total4, int accumulate) {
+    long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long step = (long)gridDim.x * blockDim.x;
+    for (; i < total4; i += step) {
+        const long at = 4 * i;
+        float4 sum = *reinterpret_cast<const float4 *>(slabs + at);
+        for (int q = 1; q < ncopies; ++q) {
+            const float4 v = *reinterpret_cast<const float4 *>(slabs + q * stride + at);
+            sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+        }
+        int k = 0;
+        long begin = 0;
+        while (k + 1 < t.count && at >= t.end[k]) begin = t.end[k++];
+        float4 *to = reinterpret_cast<float4 *>(t.dst[k] + (at - begin));
+        if (accumulate) {
+            const float4 old = *to;
+            sum.x += old.x; sum.y += old.y; sum.z += old.z; sum.w += old.w;
+        }
+        *to = sum;
+    }
+}
+
+// how many chunks the slabs region can take (0: none)
+int plan_slab_capacity(const void *slabs, size_t slab_bytes, long slab_floats) {
+    if (!slabs || slab_floats <= 0) return 0;
+    const size_t n = slab_bytes / ((size_t)slab_floats * sizeof(float));
+    return n > 65535 ? 65535 : (int)n;
+}
+
+int plan_reduce_slabs(const float *slabs, int ncopies, long stride, const SlabTargets &t, int accumulate,
+                      hipStream_t st) {
+    const long total4 = t.end[t.count - 1] / 4;
+    long blocks = (total4 + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(plan_reduce_slabs_f32, dim3((unsigned)blocks), dim3(256), 0, st, slabs, ncopies, stride,
+                       t, total4, accumulate);
+    return check_launch("reduce_slabs");
+}
+
 }  // namespace
 }  // namespace gridnet
 

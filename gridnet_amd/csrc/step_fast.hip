@@ -41,6 +41,7 @@
 
 #include "common.h"
 #include "fast_tiles.h"
+#include "plan.h"
 #include "launch.h"
 
 namespace gridnet {
@@ -825,7 +826,7 @@ void step_bwd_fast(
     float *__restrict__ dweight, float *__restrict__ dbias, float *__restrict__ dscale,
     float *__restrict__ dx, float *__restrict__ dsum_out, int B, int M, int N, int K, int inner,
     int nblk, int nchunk, int chunk_len, int param_mode, int dx_accumulate, LnFold ln,
-    float norm_eps, float *__restrict__ qr_out) {
+    float norm_eps, float *__restrict__ qr_out, long slab_stride) {
     using TL = Tile<BS, CPT>;
     static_assert(!(NORM && (LN || RES)), "the folded LayerNorm comes without normalisation");
     extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -838,6 +839,18 @@ void step_bwd_fast(
 
     int blk, chunk;
     if (!split_block_id(blockIdx.x, nblk, nchunk, blk, chunk)) return;  // grid padding
+    if (slab_stride) {
+        // the batch of this block is split over workgroups: every chunk commits into a copy of
+        // the gradient arrays of its own (plain stores; the copies are added up afterwards)
+        const long off = chunk * slab_stride;
+        dweight += off;
+        dbias += off;
+        dscale += off;
+        if (LN) {
+            ln.dgamma += off;
+            ln.dbeta += off;
+        }
+    }
     const Place<TL, CPT, NSLOT> pl(threadIdx.x, blk, N, K);
     const Fetch<TL> fx(pl.lane, pl.p0, pl.q0, pl.r0, M, N, K);
     float *win = lds + pl.slot * slot_floats;
@@ -1757,30 +1770,47 @@ int launch_bwd_ln(const StepArgs &a, hipStream_t st) {
     // one workgroup owns the whole batch of its block (no cross-workgroup reduction of the
     // parameter gradients) as soon as the blocks alone give every CU a workgroup
     const bool whole = nblk >= device_cus();
-    const Plan p = make_plan(a, NSLOT, per_cu * device_cus(), whole);
+    Plan p = make_plan(a, NSLOT, per_cu * device_cus(), whole);
     const bool new_params = (a.flags & GRIDNET_OVERWRITE_PARAMS) != 0;
-    int param_mode = kParamAtomic;
-    if (p.nchunk == 1) {
-        param_mode = new_params ? kParamStore : kParamAddExclusive;
-    } else if (new_params) {
-        if (int rc = fill_zero((float *)a.dweight, 27 * cells, st)) return rc;
-        if (int rc = fill_zero((float *)a.dbias, cells, st)) return rc;
-        if (int rc = fill_zero((float *)a.dscale, cells, st)) return rc;
-        if (LN) {
-            if (int rc = fill_zero(a.ln.dgamma, cells, st)) return rc;
-            if (int rc = fill_zero(a.ln.dbeta, cells, st)) return rc;
-        }
+    // A split batch: every chunk gets a copy of the gradient arrays in the scratch; with less
+    // room than chunks the batch is split less (down to not at all).
+    const long slab_floats = kStepSlabPlanes * cells;
+    if (p.nchunk > 1) {
+        const int room = plan_slab_capacity(a.slabs, a.slab_bytes, slab_floats);
+        if (room < p.nchunk) p = make_plan(a, NSLOT, (room < 2 ? 1 : room) * nblk, room < 2);
+    }
+    const bool split = p.nchunk > 1;
+    const int param_mode = split || new_params ? kParamStore : kParamAddExclusive;
+    float *slab = (float *)a.slabs;
+    LnFold ln = a.ln;
+    if (split && LN) {
+        ln.dgamma = slab + 29 * cells;
+        ln.dbeta = slab + 30 * cells;
     }
     const int dx_accumulate = (a.flags & GRIDNET_OVERWRITE_DX) ? 0 : 1;
     // NORM: (Q, R) per (element, block), behind the D tensor in the workspace
     float *qr = NORM ? (float *)a.workspace + (size_t)a.B * cells : nullptr;
     hipLaunchKernelGGL(kern, dim3(padded_grid(p.nblk, p.nchunk)), dim3(TL::TPS * NSLOT), lds, st,
                        (const float *)a.weight, (const float *)a.bias, (const float *)a.scale,
-                       (const float *)a.x, (const float *)a.dy, (float *)a.dweight, (float *)a.dbias,
-                       (float *)a.dscale, (float *)a.dx, (float *)a.workspace, a.B, a.M, a.N, a.K,
-                       a.inner, p.nblk, p.nchunk, p.chunk_len, param_mode, dx_accumulate, a.ln,
-                       (float)a.eps, qr);
+                       (const float *)a.x, (const float *)a.dy, split ? slab : (float *)a.dweight,
+                       split ? slab + 27 * cells : (float *)a.dbias,
+                       split ? slab + 28 * cells : (float *)a.dscale, (float *)a.dx,
+                       (float *)a.workspace, a.B, a.M, a.N, a.K, a.inner, p.nblk, p.nchunk, p.chunk_len,
+                       param_mode, dx_accumulate, ln, (float)a.eps, qr, split ? slab_floats : 0L);
     if (int rc = check_launch("step_bwd_fast")) return rc;
+    if (split) {
+        SlabTargets t{};
+        t.dst[0] = (float *)a.dweight; t.end[0] = 27 * cells;
+        t.dst[1] = (float *)a.dbias;   t.end[1] = 28 * cells;
+        t.dst[2] = (float *)a.dscale;  t.end[2] = 29 * cells;
+        t.count = 3;
+        if (LN) {
+            t.dst[3] = a.ln.dgamma; t.end[3] = 30 * cells;
+            t.dst[4] = a.ln.dbeta;  t.end[4] = 31 * cells;
+            t.count = 5;
+        }
+        if (int rc = plan_reduce_slabs(slab, p.nchunk, slab_floats, t, new_params ? 0 : 1, st)) return rc;
+    }
     // same blocks, same batch chunks; the parameter gradients are complete, dx is not yet
     constexpr int XSLOT = BS == 8 ? kCrossSlots8 : kCrossSlots4;
     constexpr int XE = BS == 8 ? kCrossElems8 : kCrossElems4;
@@ -1884,6 +1914,19 @@ size_t step_fast_backward_workspace(const StepArgs &a) {
     // normalize, two more numbers per (element, block)
     const size_t nblk = (size_t)(a.M / a.block_size) * (a.N / a.block_size) * (a.K / a.block_size);
     return ((size_t)a.B * a.M * a.N * a.K + (a.normalize ? (size_t)a.B * nblk * 2 : 0)) * sizeof(float);
+}
+
+size_t step_fast_slab_bytes(const StepArgs &a) {
+    // the most chunks any plan of the backward kernels makes: resident workgroups (two per CU with
+    // 8^3 blocks, bounded by 16 with 4^3) over the blocks, and never more than the batch gives
+    const long nblk = (long)(a.M / a.block_size) * (a.N / a.block_size) * (a.K / a.block_size);
+    if (nblk >= device_cus()) return 0;  // one workgroup owns the whole batch of its block
+    const int nslot = a.block_size == 8 ? kBwdSlots8 : kBwdSlots4;
+    long chunks = (long)(a.block_size == 8 ? 2 : 16) * device_cus() / nblk;
+    const long most = (a.B + nslot - 1) / nslot;
+    if (chunks > most) chunks = most;
+    if (chunks < 2) return 0;
+    return (size_t)chunks * kStepSlabPlanes * a.M * a.N * a.K * sizeof(float);
 }
 
 int step_forward_fast(const StepArgs &a, hipStream_t st) { return dispatch<false>(a, st); }

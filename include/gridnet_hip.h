@@ -85,7 +85,13 @@ int gridnet_hip_forward(int dtype, const void *weight, const void *bias, const v
                         void *stream);
 
 /*
- * Scratch needed by gridnet_hip_backward for this problem (bytes, may be 0).
+ * Scratch that gridnet_hip_backward wants for this problem (bytes, may be 0).  On grids with
+ * fewer blocks than the GPU has compute units it includes room for one copy of the gradient
+ * arrays per batch chunk: the batch of a block is then split over workgroups, each leaves its
+ * share in its own copy with plain stores and the copies are added in chunk order (no atomics,
+ * the same bits on every run).  A caller may hand over less, down to B*M*N*K elements (plus two
+ * floats per block and batch element with normalize): the batch is then split less, or not at
+ * all; the results agree to rounding.
  */
 size_t gridnet_hip_backward_workspace_bytes(int dtype, int B, int M, int N, int K, int inner,
                                             int block_size, int normalize);

@@ -2,17 +2,18 @@
 allocates nothing -- against gridnet_hip_backward, both called through the C ABI.
 
 Two calls in a row on the same GPU, the second on a smaller problem (the static array keeps the
-first call's contents).  Where one workgroup owns the whole batch of its block the kernels are
-bitwise reproducible and the two entry points must agree bit for bit; on grids with fewer
-blocks than the chip has CUs the parameter gradients are summed with atomics, and the pair is
-held to the fp32 bar (rtol 1e-4 / atol 1e-5) instead.  A problem whose scratch does not fit the
-array is refused before anything is enqueued.
+first call's contents).  The kernels sum in a fixed order on every grid (on grids with fewer
+blocks than the chip has CUs each chunk of the batch leaves its gradients in a copy of its own,
+in the scratch behind the D tensor, and the copies are added in chunk order), so the two entry
+points must agree bit for bit as long as both have room for the same number of copies, which the
+cases here do.  A problem whose scratch does not fit the array is refused before anything is
+enqueued.
 """
 
 import pytest
 import torch
 
-from helpers import ATOL, RTOL, assert_close, make_acts, make_params
+from helpers import make_acts, make_params
 
 pytestmark = pytest.mark.gpu
 
@@ -64,12 +65,12 @@ def test_static_scratch_matches_workspace_entry_point_twice():
     # normalize=True the scratch also carries the two numbers per (element, block)
     want, got = call_pair((32, 32, 16), 2, 4, 3, True, "silu", seed=31)
     for name, a, b in zip(names, want, got):
-        assert_close(b, a, RTOL, ATOL, name)
-    assert torch.equal(want[3], got[3]), "dx is summed in a fixed order on every grid"
-    # and once more at 8^3 blocks on a grid of few blocks (batch split over workgroups)
+        assert torch.equal(a, b), f"{name}: static-scratch call differs from the workspace call"
+    # and once more at 8^3 blocks on a grid of few blocks (batch split over workgroups: the copies
+    # of the gradient arrays share the static array with the D tensor)
     want, got = call_pair((16, 16, 32), 5, 8, 2, False, "tanh", seed=41)
     for name, a, b in zip(names, want, got):
-        assert_close(b, a, RTOL, ATOL, name)
+        assert torch.equal(a, b), f"{name}: static-scratch call differs from the workspace call"
 
 
 def test_static_scratch_rejects_what_does_not_fit():
