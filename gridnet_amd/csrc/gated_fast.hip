@@ -12,8 +12,8 @@
 // deltas of an iteration go to two zero-haloed LDS windows and are gathered from there; what
 // crosses a block boundary depends on the iterations only through D0 = sum_i delta0_i and
 // D1 = sum_i delta1_i (the halo is frozen), which the kernel leaves for the cross-block kernel
-// of the plain step run on two weight sets.  No atomics wherever one workgroup owns the whole
-// batch of its block.
+// of the plain step run on two weight sets.  No atomics: where the batch of a block is split over
+// workgroups every chunk commits into a copy of the gradient arrays of its own (see plan.h).
 
 #include "common.h"
 #include "fast_tiles.h"

@@ -52,8 +52,10 @@ def test_step_with_tensors_at_odd_addresses(bs, normalize, dtype):
     got = step_call(odd, w, b, r, x, gy, inner, bs, normalize, "silu")
     for name, g, e in zip(("y", "dweight", "dbias", "dscale", "dx"), got, want):
         assert torch.isfinite(g).all(), name
-        # same kernels, same order of operations wherever no atomics are involved
-        assert_close(g.cpu(), e.cpu(), what=name)
+        if dtype == torch.float32:  # same kernels, same order of operations: same bits
+            assert torch.equal(g.cpu(), e.cpu()), name
+        else:  # the fp64 kernels scatter with atomics
+            assert_close(g.cpu(), e.cpu(), what=name)
 
 
 @pytest.mark.parametrize("bs", [8, 4])

@@ -37,7 +37,7 @@ CASES = [
     ((64, 64, 64), 8, 4, 32, "leaky_relu", 1.0),
     # bs=4 at the C5 grid (4096 blocks), batch trimmed, its 8 inner iterations (contractive weights)
     ((64, 64, 64), 4, 8, 6, "leaky_relu", 0.5),
-    # fewer blocks than CUs: the batch is split over workgroups, parameter gradients by atomics
+    # fewer blocks than CUs: the batch is split over workgroups, one copy of the gradient arrays each
     ((32, 16, 24), 8, 3, 37, "silu", 1.0),
     ((16, 16, 16), 4, 2, 129, "tanh", 1.0),
     # a single sample, and a long thin grid
@@ -95,7 +95,7 @@ def test_tuned_fp32_against_generic_fp64_normalized(shape, bs, inner, batch):
 @pytest.mark.parametrize("shape,bs,inner,batch", [
     ((64, 64, 64), 8, 4, 32),   # one workgroup of 512 threads per block owns the whole batch
     ((64, 64, 64), 4, 3, 5),    # 4096 blocks, two 64-thread slots per workgroup
-    ((24, 40, 16), 8, 2, 70),   # fewer blocks than CUs: batch split, parameter gradients by atomics
+    ((24, 40, 16), 8, 2, 70),   # fewer blocks than CUs: batch split, one copy of the gradient arrays per chunk
 ])
 def test_gated_tuned_fp32_against_generic_fp64(shape, bs, inner, batch):
     """The gated variant at full size (tanh, the activation the reference's scripts pair it with)."""

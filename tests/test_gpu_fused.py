@@ -170,11 +170,8 @@ def test_fused_residual_chain_matches_oracle(name, grid, batch, outer, activatio
     assert torch.equal(d["grad_out"].cpu(), t["grad_out"]), "the upstream gradient was modified"
     # twice the same result: nothing is left over from one call to the next
     again = (run.forward(d["x0"]).clone(), *[g.clone() for g in run.backward(d["grad_out"])])
-    # (parameter gradients of a batch split over workgroups are summed with float atomics, whose
-    # order varies from run to run)
     for name_, a, e in zip(NAMES, again, got):
-        assert_close(a, e, rtol=1e-5, atol=1e-6 if name_ in ("y", "dx0") else summed,
-                     what=f"{name_}, second run")
+        assert torch.equal(a, e), f"{name_}: second run differs"
 
 
 @pytest.mark.parametrize("shape", [(8, 16, 24), (24, 8, 16)])
@@ -228,7 +225,7 @@ def test_fused_full_size_agrees_with_op_by_op_chain():
 
 
 @pytest.mark.parametrize("shape,batch,inner,outer,activation", [
-    ((16, 16, 16), 3, 1, 3, "silu"),       # 8 blocks: batch split over workgroups, atomics
+    ((16, 16, 16), 3, 1, 3, "silu"),       # 8 blocks: batch split over workgroups, gradient copies
     ((8, 24, 16), 5, 2, 2, "tanh"),        # non-cubic, a single block along M (no neighbour there)
     ((24, 8, 8), 1, 3, 4, "silu"),         # one sample, blocks in a row
     ((16, 32, 24), 7, 4, 3, "silu"),

@@ -1,8 +1,8 @@
 """Seeded random sweep over shapes the hand-picked cases leave out.
 
 The tuned fp32 kernels choose their launch plan from the shape (batch chunks per workgroup,
-slots per workgroup, whether a workgroup owns the whole batch of its block, atomics or plain
-stores for the parameter gradients), so a fixed list of cases exercises a fixed set of plans.
+slots per workgroup, whether a workgroup owns the whole batch of its block or the gradient arrays
+get a copy per batch chunk), so a fixed list of cases exercises a fixed set of plans.
 Here grid, block size, batch, inner iterations, activation and the accumulate/overwrite flags are
 drawn at random (fixed seeds) and every draw is held to the generic kernels run in fp64 on the
 same fp32 inputs -- the two share no device code, and each is held to the CPU oracle elsewhere
