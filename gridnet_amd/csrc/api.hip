@@ -100,7 +100,7 @@ using namespace gridnet;
 
 extern "C" {
 
-int gridnet_hip_version(void) { return 5; }  // 2: fused body; 3: residual forward and backward; 4: gated backward takes a workspace; 5: backward on static scratch
+int gridnet_hip_version(void) { return 6; }  // 2: fused body; 3: residual forward and backward; 4: gated backward takes a workspace; 5: backward on static scratch; 6: chain backward, probe, gradient copies for split batches
 
 const char *gridnet_hip_last_error(void) { return error_buffer(); }
 
