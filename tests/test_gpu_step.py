@@ -244,3 +244,21 @@ def test_largest_grid_the_index_range_allows(bs):
     del w, dw, leaves, y
     gc.collect()
     torch.cuda.empty_cache()
+
+
+def test_machine_ceiling_probes_report_sane_figures():
+    """gridnet_hip_probe (the figures bench.py quotes beside the vendor peaks): every quantity comes
+    back positive and below what the part can do; an unknown quantity is refused."""
+    import ctypes
+
+    from gridnet_amd import native as n
+
+    fma, lds, clock, copy = (n.probe(k) for k in ("fma_tfma_per_s", "lds_gb_per_s", "clock_ghz", "copy_gb_per_s"))
+    print(f"probes: {fma:.1f} TFMA/s, LDS {lds:.0f} GB/s, {clock:.2f} GHz, copy {copy:.0f} GB/s", flush=True)
+    assert 5.0 < fma < 80.0         # 39.3 TFMA/s is the unpacked fp32 peak of 256 CUs at 2.4 GHz
+    assert 1.0e4 < lds < 4.0e5
+    assert 0.5 < clock < 3.5
+    assert 500.0 < copy < 8000.0    # read + write against 8 TB/s
+    out = ctypes.c_double(0.0)
+    assert n.lib.gridnet_hip_probe(99, ctypes.byref(out)) != 0
+    assert "unknown" in n.last_error()
