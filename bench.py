@@ -262,6 +262,7 @@ def main():
     # ceilings of this machine, measured now by the library's probe kernels
     from gridnet_amd import native
     ceil = {k: native.probe(k) for k in native.PROBES}
+    lds_widths = {k: native.probe(k) for k in native.LDS_WIDTH_PROBES}
     lds_peak = LDS_BYTES_PER_CLOCK_PER_CU * CUS * ceil["clock_ghz"]
     dom_s = kernel_s[dominant]
     achieved = bytes_[dominant] / dom_s / 1e9
@@ -316,6 +317,7 @@ def main():
                 "busy_frac": counters.get("lds_busy_frac"),
                 "bank_conflict_frac_of_busy": counters.get("lds_conflict_frac_of_busy"),
                 "measured_read_ceiling": ceil["lds_gb_per_s"],
+                "pipe_cycles_per_wave_read": lds_widths,
                 "peak_is": "128 B per clock and CU x 256 CUs x the measured core clock; 16-byte reads go "
                            "beyond it on this part, see measured_read_ceiling"},
         "machine": {"core_clock_ghz_under_load": ceil["clock_ghz"],

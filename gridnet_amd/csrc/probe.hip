@@ -67,6 +67,45 @@ __global__ __launch_bounds__(kProbeThreads) void probe_clock(float *out, long lo
     }
 }
 
+// One workgroup of 8 waves on one CU: cycles of the CU's LDS pipe per wave-level read instruction of
+// a given width, lanes at consecutive addresses (no bank conflicts).  W: 1, 2, 4 = 32-, 64-, 128-bit
+// reads; 22 = two 64-bit reads that the compiler fuses into one two-address instruction.
+template <int W>
+__global__ __launch_bounds__(512) void probe_lds_width(float *out, long long *ticks, int trips) {
+    __shared__ __attribute__((aligned(16))) float lds[16384];
+    for (int i = threadIdx.x; i < 16384; i += 512) lds[i] = i * 1e-4f;
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    // the pair of 64-bit reads as the backward kernels issue it: four floats from an 8-byte-aligned
+    // address, neighbouring lanes two floats apart (their rows overlap)
+    const int at = W == 22 ? lane * 2 : lane * W;
+    float acc = 0.f;
+    __syncthreads();
+    const long long c0 = clock64();
+    for (int t = 0; t < trips; ++t) {
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const float *p = lds + at + ((u + t) & 7) * 1024;
+            if (W == 4) {
+                const float4 q = *reinterpret_cast<const float4 *>(p);
+                acc += q.x + q.y + q.z + q.w;
+            } else if (W == 2) {
+                const float2 q = *reinterpret_cast<const float2 *>(p);
+                acc += q.x + q.y;
+            } else if (W == 22) {
+                const float2 q = *reinterpret_cast<const float2 *>(p);
+                const float2 r = *reinterpret_cast<const float2 *>(p + 2);
+                acc += q.x + q.y + r.x + r.y;
+            } else {
+                acc += p[0];
+            }
+        }
+    }
+    const long long c1 = clock64();
+    out[threadIdx.x] = acc;
+    if (lane == 0) ticks[threadIdx.x / 64] = c1 - c0;
+}
+
 __global__ __launch_bounds__(kProbeThreads) void probe_copy(const float4 *src, float4 *dst, size_t n) {
     size_t i = (size_t)blockIdx.x * kProbeThreads + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * kProbeThreads;
@@ -150,6 +189,29 @@ extern "C" int gridnet_hip_probe(int what, double *result) {
         hipLaunchKernelGGL(probe_copy, dim3(cus * 16), dim3(kProbeThreads), 0, 0, dst, src, n);  // first touch
         s = timer.best(4, [&] { hipLaunchKernelGGL(probe_copy, dim3(cus * 16), dim3(kProbeThreads), 0, 0, src, dst, n); });
         if (s > 0) *result = 2.0 * (double)n * sizeof(float4) / s / 1e9;
+        break;
+    }
+    case GRIDNET_PROBE_LDS_B32:
+    case GRIDNET_PROBE_LDS_B64:
+    case GRIDNET_PROBE_LDS_B128:
+    case GRIDNET_PROBE_LDS_2XB64: {  // LDS-pipe cycles per wave-level read instruction
+        if (hipMalloc(&ticks, 8 * sizeof(long long)) != hipSuccess) { rc = fail(GRIDNET_ERR_LAUNCH, "probe: hipMalloc failed"); break; }
+        const int trips = 2000;
+        double best = -1.0;
+        for (int rep = 0; rep < 3; ++rep) {
+            if (what == GRIDNET_PROBE_LDS_B32) hipLaunchKernelGGL(probe_lds_width<1>, dim3(1), dim3(512), 0, 0, out, ticks, trips);
+            else if (what == GRIDNET_PROBE_LDS_B64) hipLaunchKernelGGL(probe_lds_width<2>, dim3(1), dim3(512), 0, 0, out, ticks, trips);
+            else if (what == GRIDNET_PROBE_LDS_B128) hipLaunchKernelGGL(probe_lds_width<4>, dim3(1), dim3(512), 0, 0, out, ticks, trips);
+            else hipLaunchKernelGGL(probe_lds_width<22>, dim3(1), dim3(512), 0, 0, out, ticks, trips);
+            long long h[8] = {0};
+            if (hipDeviceSynchronize() != hipSuccess ||
+                hipMemcpy(h, ticks, sizeof(h), hipMemcpyDeviceToHost) != hipSuccess) { best = -1.0; break; }
+            long long mx = 0;
+            for (int w = 0; w < 8; ++w) mx = h[w] > mx ? h[w] : mx;
+            const double per = (double)mx / (trips * 8.0 * 8.0);  // 8 reads per trip, 8 waves share the pipe
+            if (best < 0 || per < best) best = per;
+        }
+        if (best > 0) { *result = best; s = 1.0; }
         break;
     }
     default:

@@ -123,12 +123,15 @@ except AttributeError as exc:  # an older build of the library without some entr
 
 
 PROBES = {"fma_tfma_per_s": 0, "lds_gb_per_s": 1, "clock_ghz": 2, "copy_gb_per_s": 3}  # GRIDNET_PROBE_*
+# LDS-pipe cycles per wave-level read instruction, by width (GRIDNET_PROBE_LDS_B32 ... _2XB64)
+LDS_WIDTH_PROBES = {"ds_read_b32": 4, "ds_read_b64": 5, "ds_read_b128": 6, "ds_read2_b64": 7}
 
 
 def probe(what: str) -> float:
     """One of the machine ceilings of gridnet_hip_probe on the current device."""
     out = ctypes.c_double(0.0)
-    check(lib.gridnet_hip_probe(PROBES[what], ctypes.byref(out)))
+    kind = PROBES[what] if what in PROBES else LDS_WIDTH_PROBES[what]
+    check(lib.gridnet_hip_probe(kind, ctypes.byref(out)))
     return out.value
 
 

@@ -304,8 +304,13 @@ int gridnet_hip_chain_backward(int dtype, const void *weight, const void *bias, 
  *   GRIDNET_PROBE_LDS    conflict-free 16-byte LDS reads over all CUs, GB/s
  *   GRIDNET_PROBE_CLOCK  core clock while every CU runs the FMA loop, GHz
  *   GRIDNET_PROBE_COPY   device-to-device copy of 1 GiB by a plain kernel, read + write GB/s
+ *   GRIDNET_PROBE_LDS_B32 / _B64 / _B128 / _2XB64   cycles of one CU's LDS pipe per wave-level read
+ *                        instruction of that width (2XB64: one two-address 64-bit read), lanes at
+ *                        consecutive addresses, 8 waves
  */
-enum { GRIDNET_PROBE_FMA = 0, GRIDNET_PROBE_LDS = 1, GRIDNET_PROBE_CLOCK = 2, GRIDNET_PROBE_COPY = 3 };
+enum { GRIDNET_PROBE_FMA = 0, GRIDNET_PROBE_LDS = 1, GRIDNET_PROBE_CLOCK = 2, GRIDNET_PROBE_COPY = 3,
+       GRIDNET_PROBE_LDS_B32 = 4, GRIDNET_PROBE_LDS_B64 = 5, GRIDNET_PROBE_LDS_B128 = 6,
+       GRIDNET_PROBE_LDS_2XB64 = 7 };
 int gridnet_hip_probe(int what, double *result);
 
 #ifdef __cplusplus

@@ -259,6 +259,10 @@ def test_machine_ceiling_probes_report_sane_figures():
     assert 1.0e4 < lds < 4.0e5
     assert 0.5 < clock < 3.5
     assert 500.0 < copy < 8000.0    # read + write against 8 TB/s
+    widths = {k: n.probe(k) for k in n.LDS_WIDTH_PROBES}
+    print("LDS pipe cycles per wave-level read:", {k: round(v, 2) for k, v in widths.items()}, flush=True)
+    assert all(1.0 < v < 64.0 for v in widths.values())
+    assert widths["ds_read_b32"] < widths["ds_read_b128"]
     out = ctypes.c_double(0.0)
     assert n.lib.gridnet_hip_probe(99, ctypes.byref(out)) != 0
     assert "unknown" in n.last_error()
