@@ -643,7 +643,7 @@ template <int ACT, bool DEFER> int launch_chain(const StepArgs &a, hipStream_t s
     // room than chunks the batch is split less (down to not at all).
     const long slab_floats = kStepSlabPlanes * cells;
     if (k.nchunk > 1) {
-        const int room = plan_slab_capacity(a.slabs, a.slab_bytes, slab_floats);
+        const int room = plan_split_room(plan_slab_capacity(a.slabs, a.slab_bytes, slab_floats), a.B, k.chunk_len);
         if (room < k.nchunk)
             plan_batch_chunks(a.B, k.nblk, 1, (room < 2 ? 1 : room) * k.nblk, room < 2, k.nchunk, k.chunk_len);
     }

@@ -474,7 +474,7 @@ template <int BS, int NSLOT, int ACT> int launch_bwd(const StepArgs &a, hipStrea
     // room than chunks the batch is split less (down to not at all).
     const long slab_floats = kGatedSlabPlanes * cells;
     if (nchunk > 1) {
-        const int room = plan_slab_capacity(a.slabs, a.slab_bytes, slab_floats);
+        const int room = plan_split_room(plan_slab_capacity(a.slabs, a.slab_bytes, slab_floats), a.B, chunk_len);
         if (room < nchunk) plan_chunks(a.B, nblk, NSLOT, (room < 2 ? 1 : room) * nblk, room < 2, nchunk, chunk_len);
     }
     const bool split = nchunk > 1;

@@ -1776,7 +1776,7 @@ int launch_bwd_ln(const StepArgs &a, hipStream_t st) {
     // room than chunks the batch is split less (down to not at all).
     const long slab_floats = kStepSlabPlanes * cells;
     if (p.nchunk > 1) {
-        const int room = plan_slab_capacity(a.slabs, a.slab_bytes, slab_floats);
+        const int room = plan_split_room(plan_slab_capacity(a.slabs, a.slab_bytes, slab_floats), a.B, p.chunk_len);
         if (room < p.nchunk) p = make_plan(a, NSLOT, (room < 2 ? 1 : room) * nblk, room < 2);
     }
     const bool split = p.nchunk > 1;
