@@ -305,9 +305,11 @@ template <typename TL, int NT = TL::TPS> struct Fetch {  // NT: threads of a slo
         for (int e = 0; e < RPT; ++e)
             if (loff[e] >= 0) {
                 const float end = (ok[e] && edge_ok[e]) ? v[e][HC] : 0.f;
+                int lo = loff[e];  // opaque: see commit_ln
+                asm volatile("" : "+v"(lo));
 #pragma unroll
                 for (int copy = 0; copy < COPIES; ++copy) {
-                    float *row = win + copy * TL::WIN + loff[e];
+                    float *row = win + copy * TL::WIN + lo;
                     // first half: [end, cells...]; second half: [cells..., end]
                     row[hi[e] ? HC : 0] = end;
 #pragma unroll
@@ -387,7 +389,13 @@ template <typename TL, int NT = TL::TPS> struct Fetch {  // NT: threads of a slo
                 load_cells<HC>(from, g);
                 load_cells<HC>(from + HC, b);
                 const float2 ends = *reinterpret_cast<const float2 *>(from + 2 * HC);
-                const int at_end = loff[e] + (hi[e] ? HC : 0), at_cells = loff[e] + (hi[e] ? 0 : 1);
+                // The row's place is taken through an opaque copy: the two addresses derived from
+                // it are worked out here, per element (two instructions), instead of living in
+                // registers of their own across the batch loop -- where the backward kernels have
+                // none to spare, so that they came back from scratch memory one wait at a time.
+                int lo = loff[e];
+                asm volatile("" : "+v"(lo));
+                const int at_end = lo + (hi[e] ? HC : 0), at_cells = lo + (hi[e] ? 0 : 1);
                 const float end = (ok[e] && edge_ok[e]) ? fmaf((v[e][HC] - mean) * rstd, ends.x, ends.y)
                                                         : 0.f;
                 float val[HC];

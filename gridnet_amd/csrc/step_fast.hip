@@ -547,7 +547,10 @@ void step_fwd_split(
             float wave_mean, wave_m2;  // one pair per wave
             slot_wave_moments<128>(mean, m2, 64, wave_mean, wave_m2);
             if ((pl.lane & 63) == 0) {
-                float *to = ln.y_part + (((long)s * nblk + blk) * 2 + pl.lane / 64) * 2;
+                // the wave's number as a scalar: the address is uniform then, and no per-lane
+                // pointer is carried (spilled) through the batch loop for this one store
+                const int wv = __builtin_amdgcn_readfirstlane(pl.lane / 64);
+                float *to = ln.y_part + (((long)s * nblk + blk) * 2 + wv) * 2;
                 to[0] = wave_mean;
                 to[1] = wave_m2;
             }
