@@ -27,7 +27,7 @@ LDS_BYTES_PER_CLOCK_PER_CU = 128
 CUS = 256
 
 
-def gpu_run(wl, steps, warmup, fused, graph_replay=True):
+def gpu_run(wl, steps, warmup, fused, graph_replay=True, chain_all=None):
     import torch
 
     from gridnet_amd.configs import make_inputs
@@ -38,7 +38,7 @@ def gpu_run(wl, steps, warmup, fused, graph_replay=True):
     t = {k: v.to(dev) for k, v in make_inputs(wl, seed=0).items()}
     run = BodyRunner(t["weight"], t["bias"], t["scale"], t["gamma"], t["beta"], wl.batch, wl.inner,
                      wl.outer, wl.block_size, wl.activation, wl.normalize, backward=wl.backward,
-                     fused=fused)
+                     fused=fused, chain_all=chain_all)
 
     def one_step():
         run.forward(t["x0"])
@@ -53,6 +53,11 @@ def gpu_run(wl, steps, warmup, fused, graph_replay=True):
         one_step()
     torch.cuda.synchronize()
     wall = (time.perf_counter() - t0) / steps
+    # the one-launch chain backward reports through a status word whether its bounded waits held;
+    # a timing with invalid results is no timing
+    if run.chain_all_status() != 0:
+        sys.exit("bench.py: gridnet_hip_chain_backward_all gave up (status word set): results invalid; "
+                 "re-run with --chain-all off")
 
     # The same step as one captured HIP graph, replayed: what is left when the host side (Python,
     # ctypes, launch calls) is taken out.  Reported beside the eager figure, which stays the headline.
@@ -102,7 +107,7 @@ def gpu_run(wl, steps, warmup, fused, graph_replay=True):
         assert p0 == 0 and p1 == 1
         spans.setdefault(name, []).append(e0.elapsed_time(e1) * 1e-3)
     kernel_s = {k: sum(v) / len(v) for k, v in spans.items()}
-    return wall, graph_s, kernel_s
+    return wall, graph_s, kernel_s, bool(getattr(run, "chain_all", False))
 
 
 def cpu_baseline(wl, budget_s=25.0):
@@ -225,6 +230,10 @@ def main():
     ap.add_argument("--normalize", action="store_true",
                     help="the workload with normalize=True (the reference's default, which its "
                          "training scripts switch off); op-by-op path")
+    ap.add_argument("--chain-all", choices=("auto", "on", "off"), default="auto",
+                    help="the backward of the whole chain in one launch of resident workgroups "
+                         "(gridnet_hip_chain_backward_all): where it applies and fills the chip, "
+                         "wherever it applies, never")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true",
                     help="skip the HIP graph replay (for runs under a counter-collecting profiler)")
@@ -240,7 +249,8 @@ def main():
     if args.normalize:
         wl = dataclasses.replace(wl, normalize=True, name=wl.name + " normalize")
     fused = args.path == "fused" and not wl.normalize and wl.inner >= 1
-    wall, graph_s, kernel_s = gpu_run(wl, args.steps, args.warmup, fused, not args.no_graph)
+    wall, graph_s, kernel_s, one_launch = gpu_run(wl, args.steps, args.warmup, fused, not args.no_graph,
+                                      {"auto": None, "on": True, "off": False}[args.chain_all])
     bytes_ = wl.algorithmic_bytes()
     if fused:  # a fused entry point does the work of the step AND of the LayerNorm beside it
         bytes_["step_fwd"] += bytes_["ln_fwd"]
@@ -286,7 +296,9 @@ def main():
         "data": "synthetic",
         "config": {"workload": wl.name, "activation": wl.activation, "normalize": wl.normalize,
                    "pass": "fwd+bwd" if wl.backward else "fwd",
-                   "path": "fused step+LayerNorm entry points" if fused else "step and LayerNorm calls"},
+                   "path": ("fused step+LayerNorm entry points" + (", backward of the chain in one launch"
+                                                                   if one_launch else ""))
+                           if fused else "step and LayerNorm calls"},
         "timing": {"headline": "eager wall clock over the timed steps, synchronised on both sides",
                    "eager_ms_per_step": wall * 1e3,
                    "hip_graph_replay_ms_per_step": None if graph_s is None else graph_s * 1e3},

@@ -25,6 +25,14 @@ FLAGS = [
 ]
 
 
+# per source file, on top of FLAGS
+FILE_FLAGS = {
+    # chain_bwd.hip posts an arrival with an atomic add from one lane and reads the returned count
+    # an iteration later; the atomic optimizer would make it a wave reduction that waits at once
+    "chain_bwd.hip": ["-mllvm", "-amdgpu-atomic-optimizer-strategy=None"],
+}
+
+
 def build(verbose: bool = True, extra_flags=(), out=None, objdir=None) -> str:
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     objdir = objdir or os.path.join(HERE, "build")
@@ -33,7 +41,7 @@ def build(verbose: bool = True, extra_flags=(), out=None, objdir=None) -> str:
 
     def compile_one(src):
         obj = os.path.join(objdir, src.replace(".hip", ".o"))
-        cmd = [hipcc, *FLAGS, *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [hipcc, *FLAGS, *FILE_FLAGS.get(src, []), *extra_flags, "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose:
             print(" ".join(cmd), flush=True)
         res = subprocess.run(cmd, capture_output=True, text=True)

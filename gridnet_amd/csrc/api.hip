@@ -100,7 +100,7 @@ using namespace gridnet;
 
 extern "C" {
 
-int gridnet_hip_version(void) { return 6; }  // 2: fused body; 3: residual forward and backward; 4: gated backward takes a workspace; 5: backward on static scratch; 6: chain backward, probe, gradient copies for split batches
+int gridnet_hip_version(void) { return 7; }  // 2: fused body; 3: residual forward and backward; 4: gated backward takes a workspace; 5: backward on static scratch; 6: chain backward, gradient copies for split batches; 7: whole chain in one launch
 
 const char *gridnet_hip_last_error(void) { return error_buffer(); }
 
@@ -576,6 +576,70 @@ int gridnet_hip_chain_backward(int dtype, const void *weight, const void *bias, 
     const int nblk = (M / block_size) * (N / block_size) * (K / block_size);
     return layernorm_finalize_sums(a.ln.x_part, nblk * step_fast_backward_parts(block_size),
                                    (long)M * N * K, (float *)x_sums, B, st);
+}
+
+static int chain_spin_limit = 200000;
+
+int gridnet_hip_chain_set_spin_limit(int limit) {
+    const int old = chain_spin_limit;
+    chain_spin_limit = limit;
+    return old;
+}
+
+int gridnet_hip_chain_all_supported(int dtype, int B, int M, int N, int K, int inner, int outer,
+                                    int block_size, int normalize) {
+    if (dtype != GRIDNET_F32 || block_size != 8 || normalize) return 0;
+    return chain_all_supports(B, M, N, K, inner, outer) ? 1 : 0;
+}
+
+size_t gridnet_hip_chain_all_workspace_bytes(int B, int M, int N, int K, int inner, int outer,
+                                             int block_size) {
+    if (B <= 0 || M <= 0 || N <= 0 || K <= 0 || outer <= 0 || block_size != 8 || M % 8 || N % 8 || K % 8)
+        return 0;
+    ChainAll c{};
+    c.B = B; c.M = M; c.N = N; c.K = K; c.inner = inner; c.outer = outer;
+    return chain_all_workspace(c);
+}
+
+int gridnet_hip_chain_backward_all(int dtype, const void *weight, const void *bias, const void *scale,
+                                   const void *gamma, const void *beta, const void *x0,
+                                   const void *y_raw, const void *stats, const void *dy,
+                                   void *dweight, void *dbias, void *dscale, void *dgamma,
+                                   void *dbeta, void *dx, int B, int M, int N, int K, int inner,
+                                   int outer, int block_size, int activation, int flags,
+                                   void *workspace, size_t workspace_bytes, void *stream) {
+    StepArgs a{};
+    a.dtype = dtype; a.weight = weight; a.bias = bias; a.scale = scale; a.x = x0; a.dy = dy;
+    a.dweight = dweight; a.dbias = dbias; a.dscale = dscale; a.dx = dx;
+    a.B = B; a.M = M; a.N = N; a.K = K; a.inner = inner; a.block_size = block_size;
+    a.activation = activation;
+    if (dtype != GRIDNET_F32 || block_size != 8)
+        return fail(GRIDNET_ERR_ARGUMENT, "the one-launch chain is float32 with block_size 8 (dtype id %d, block_size %d)",
+                    dtype, block_size);
+    if (int rc = check_step(a, true)) return rc;
+    if (!chain_all_supports(B, M, N, K, inner, outer))
+        return fail(GRIDNET_ERR_ARGUMENT,
+                    "the one-launch chain does not cover this problem (B=%d grid %dx%dx%d inner=%d outer=%d): "
+                    "see gridnet_hip_chain_all_supported; use gridnet_hip_chain_backward",
+                    B, M, N, K, inner, outer);
+    if (!gamma || !beta || !y_raw || !stats || !dgamma || !dbeta)
+        return fail(GRIDNET_ERR_ARGUMENT, "null pointer");
+    ChainAll c{};
+    c.weight = (const float *)weight; c.bias = (const float *)bias; c.scale = (const float *)scale;
+    c.gamma = (const float *)gamma; c.beta = (const float *)beta;
+    c.x0 = (const float *)x0; c.y_raw = (const float *)y_raw; c.stats = (const float *)stats;
+    c.dy = (const float *)dy;
+    c.dweight = (float *)dweight; c.dbias = (float *)dbias; c.dscale = (float *)dscale;
+    c.dgamma = (float *)dgamma; c.dbeta = (float *)dbeta; c.dx = (float *)dx;
+    c.B = B; c.M = M; c.N = N; c.K = K; c.inner = inner; c.outer = outer;
+    c.activation = activation; c.flags = flags;
+    c.workspace = workspace; c.workspace_bytes = workspace_bytes;
+    c.spin_limit = chain_spin_limit;
+    const size_t need = chain_all_workspace(c);
+    if (!workspace || workspace_bytes < need)
+        return fail(GRIDNET_ERR_WORKSPACE, "the one-launch chain needs %zu bytes of workspace, got %zu", need,
+                    workspace ? workspace_bytes : (size_t)0);
+    return chain_backward_all(c, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -112,7 +112,40 @@ struct ChainBwdArgs {
     float *x_part;             // DEFER: [B, nblk, 2] sums for the LayerNorm in front of this step
     int B, M, N, K, inner, nblk, nchunk, chunk_len, param_mode;
     long slab_stride;          // split batch: floats between the chunks' copies of the gradient arrays, else 0
+    // ---- ALL: every step of the chain in one launch (see chain_bwd) ----
+    // y_raw and y_stats then point at step 0's and the steps lie step_floats / 2 B floats apart;
+    // dy is the gradient handed to the last step; x, x_stats, y_sums, halo_in, dx, out2 are unused.
+    const float *x0;           // input of step 0 (no LayerNorm in front of it)
+    float *sums;               // [steps * B][2] by item: the LayerNorm sums an item asks for; those of
+                               // the last step's items are given, the others are formed here
+    float *dx_even, *dx_odd;      // step j leaves the block-local part of its input gradient in the one of its parity
+    float *halo_even, *halo_odd;  // ... and what crosses block boundaries
+    unsigned *status;          // one word, zero on entry: set when a bounded wait ran out
+    unsigned *arrive, *ready;  // by item, (steps - 1) * B each, zero on entry
+    int steps, spin_limit;     // spin_limit < 0: never publish (the give-up path under test), limit = -spin_limit
+    long step_floats;          // floats between y_raw of consecutive steps
 };
+
+// Coherent accesses for data that workgroups on other XCDs write or read WHILE THE KERNEL RUNS:
+// relaxed atomics at agent scope compile to loads and stores that bypass the XCD-private L2
+// (write-through stores, loads that do not hit a stale line); plain accesses only see other
+// XCDs' writes across a kernel boundary.
+template <typename T> __device__ __forceinline__ T ld_agent(const T *p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename T> __device__ __forceinline__ void st_agent(T *p, T v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float2 ld_agent2(const float *p) {
+    const unsigned long long u = ld_agent(reinterpret_cast<const unsigned long long *>(p));
+    return make_float2(__uint_as_float((unsigned)u), __uint_as_float((unsigned)(u >> 32)));
+}
+// the same word for every lane, loaded as a vector load (see load_ahead)
+template <typename T> __device__ __forceinline__ T ld_agent_uniform(const T *p) {
+    int zero;
+    asm volatile("v_mov_b32 %0, 0" : "=v"(zero));
+    return ld_agent(p + zero);
+}
 
 // LDS (floats): [x window x2 | delta window x2 | u_i of the owned cells, inner slabs of 512 |
 // gamma, beta of the window, packed | sums of the four waves | weights of the shell entries
@@ -135,9 +168,30 @@ __device__ __forceinline__ int stride_of(unsigned code) {
     return code == 0 ? 1 : code == 1 ? ChainTile::RS : ChainTile::PS;
 }
 
-template <int ACT, bool DEFER>
+// ALL: one launch walks every step of the chain, last to first.  A workgroup keeps its block for the
+// whole chain: the weights, the mirrored weights, the tables and -- with one parameter set shared
+// by the steps -- the gradient accumulators stay where they are from step to step (no set-up,
+// no drain, no read-modify-write of the gradient arrays per step), and nobody waits for the
+// slowest workgroup of a step.  The workgroups must all be resident (cooperative launch).
+// What step j-1 needs of step j for batch element s -- the values its neighbours' blocks send
+// across the block boundaries and the two per-sample sums of the LayerNorm between the steps,
+// which every block contributes to -- travels through memory behind a counter per (step,
+// element): a workgroup adds 1 once its stores for the pair have been acknowledged.  Pair number m
+// has a workgroup in charge, m modulo the number of workgroups -- NOT the last one to arrive: that
+// is the slowest workgroup of the moment every time, and the extra work would keep it the
+// slowest (measured: one workgroup fell 25 % behind and the whole grid followed at its pace).
+// The one in charge looks at the counter once per iteration; when it reads the number of blocks
+// it sums the blocks' shares in block order (always the same bits), stores the two means and
+// then sets the pair's ready word.
+// A workgroup looks at that word before it requests the pair's data for step j-1.  By then the
+// pair is a whole batch old, so the look normally costs nothing: the word is requested an
+// element ahead, together with the window.  Waits are bounded: a wave that runs out of tries
+// sets the status word and stops waiting for good (results are then invalid, the host falls
+// back to one launch per step), so every workgroup reaches the end whatever happens.
+template <int ACT, bool DEFER, bool ALL = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 void chain_bwd(const ChainBwdArgs a) {
+    static_assert(DEFER || !ALL, "inside one launch every step hands its halo values on");
     using TL = ChainTile;
     constexpr int BS = 8, CPT = 2, NC = BS * BS * BS;
     extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -167,7 +221,7 @@ void chain_bwd(const ChainBwdArgs a) {
     const Fetch<TL> fx(tid, pl.p0, pl.q0, pl.r0, a.M, a.N, a.K);
     const long cells = (long)a.M * a.N * a.K;
     const int N = a.N, K = a.K;
-    const bool ln_in = a.x_stats != nullptr;
+    const bool ln_in = ALL || a.x_stats != nullptr;  // ALL: every step but the first
     // the x window copy that would receive x_inner (never needed) gets zeros in the block's cells
     // instead: the window's halo alone, for the weights of the taps that read it
     const float *xhalo = win + (inner & 1) * TL::WIN;
@@ -291,10 +345,10 @@ void chain_bwd(const ChainBwdArgs a) {
     // ---- what this thread's cells receive from the blocks around: where, and whether ----
     const int fi = pl.i == 0 ? 0 : pl.i == BS - 1 ? 1 : -1, fj = pl.j == 0 ? 0 : pl.j == BS - 1 ? 1 : -1,
               fk = pl.kt == 0 ? 0 : pl.kt == TL::KT - 1 ? 1 : -1;
-    const bool have_in = a.halo_in != nullptr;
-    const bool ei = have_in && (fi == 0 ? bi > 0 : fi == 1 ? bi < mb - 1 : false);
-    const bool ej = have_in && (fj == 0 ? bj > 0 : fj == 1 ? bj < nb - 1 : false);
-    const bool ek = have_in && (fk == 0 ? bk > 0 : fk == 1 ? bk < kb - 1 : false);
+    const bool have_in = ALL || a.halo_in != nullptr;  // ALL: every step but the last, see the loop
+    const bool ei0 = have_in && (fi == 0 ? bi > 0 : fi == 1 ? bi < mb - 1 : false);
+    const bool ej0 = have_in && (fj == 0 ? bj > 0 : fj == 1 ? bj < nb - 1 : false);
+    const bool ek0 = have_in && (fk == 0 ? bk > 0 : fk == 1 ? bk < kb - 1 : false);
     {
         const int zi = max(fi, 0), zj = max(fj, 0), zk = max(fk, 0), k2 = pl.kt * CPT;
         const unsigned o[7] = {unsigned(kSegI + zi * 64 + pl.j * 8 + k2), unsigned(kSegJ + zj * 64 + pl.i * 8 + k2),
@@ -306,8 +360,8 @@ void chain_bwd(const ChainBwdArgs a) {
         tab(kTabIn + 2) = o[6];
     }
     // without halo_in every flag is off and the (unconditional) loads read dy instead: in bounds
-    const float *hin = have_in ? a.halo_in : a.dy;
-    const float *xst = ln_in ? a.x_stats : a.y_stats;
+    const float *hin = ALL ? nullptr : have_in ? a.halo_in : a.dy;
+    const float *xst = ALL ? nullptr : ln_in ? a.x_stats : a.y_stats;
     const unsigned ugc = 4u * pl.gc;  // byte offset of the owned cells within a sample
 
     typename Fetch<TL>::Buf pre;
@@ -342,15 +396,40 @@ void chain_bwd(const ChainBwdArgs a) {
         acc_ref(6 + c) = dbet[c];
     }
 
-    const int s0 = chunk * a.chunk_len, s1 = min(a.B, s0 + a.chunk_len);
+    const int s0 = ALL ? 0 : chunk * a.chunk_len, s1 = ALL ? a.B : min(a.B, s0 + a.chunk_len);
+    // ALL: the walk is last step first, the elements of a step in order: item n is element n % B of
+    // step steps - 1 - n / B.  Counters, ready words and LayerNorm sums are numbered by item.  What
+    // depends on the step alone is kept in (scalar) variables that change once per step.
+    const int items = ALL ? a.steps * a.B : s1 - s0;
+    const int counted = ALL ? (a.steps - 1) * a.B : 0;  // the items of every step but the first hand something on
+    const float *c_dy = a.dy, *c_rec = hin, *c_yr = a.y_raw, *c_ystat = a.y_stats;  // the element's gradient,
+                                                       // what the blocks around left for it, its raw output
+    const float *c_x = a.x, *c_xst = xst;              // the step's input and its statistics
+    float *c_dxo = a.dx, *c_halo = a.out2;             // where the step leaves dx and its halo values
+    bool c_later = true, c_ln = ln_in;                 // a later step exists; the input passes a LayerNorm
+    auto enter_step = [&](int jj) {
+        const bool odd = (jj & 1) != 0;
+        c_later = jj < a.steps - 1;
+        c_dy = c_later ? (odd ? a.dx_even : a.dx_odd) : a.dy;
+        c_rec = c_later ? (odd ? a.halo_even : a.halo_odd) : a.dy;  // no later step: every flag is off
+        c_yr = a.y_raw + jj * a.step_floats;
+        c_ystat = a.y_stats + (long)jj * 2 * a.B;
+        c_ln = jj > 0;
+        c_x = c_ln ? a.y_raw + (jj - 1) * a.step_floats : a.x0;
+        c_xst = a.y_stats + (long)(c_ln ? jj - 1 : 0) * 2 * a.B;
+        c_dxo = odd ? a.dx_odd : a.dx_even;
+        c_halo = odd ? a.halo_odd : a.halo_even;
+    };
     float nxm = 0.f, nxr = 1.f;  // LayerNorm statistics of the element in `pre`
-    auto fetch_window = [&](int s) {
-        fx.fetch(a.x + (long)s * cells, pre);
-        nxm = load_ahead(xst, 2 * s);
-        nxr = load_ahead(xst, 2 * s + 1);
+    bool nx_ln = ln_in;          // ... and whether it passes a LayerNorm on the way in
+    auto fetch_window = [&](const float *xs, const float *st, bool ln, int s) {
+        nx_ln = ln;
+        fx.fetch(xs + (long)s * cells, pre);
+        nxm = load_ahead(st, 2 * s);
+        nxr = load_ahead(st, 2 * s + 1);
     };
     auto commit_window = [&]() {
-        if (ln_in) fx.commit_ln(win, pre, affine, nxm, nxr);
+        if (nx_ln) fx.commit_ln(win, pre, affine, nxm, nxr);
         else fx.commit(win, pre);
     };
     // An element is finished one element late.  Its dx is stored behind the requests of the element
@@ -363,10 +442,12 @@ void chain_bwd(const ChainBwdArgs a) {
     float g_done[CPT], o_done[2];     // o_done: the element's D (without deferred halos)
     float t1_done = 0.f, t2_done = 0.f, nh_done[2] = {0.f, 0.f};  // its LayerNorm sums so far; x-hat at the shell entries
     int done_s = -1, sums_s = -1;
+    // ALL: where the step of the finished element leaves its results
+    float *d_dxo = a.dx, *d_halo = a.out2;
     auto store_done = [&]() {
         if (done_s < 0) return;
         const long o = (long)done_s * cells;
-        at_bytes<float2>(a.dx + o, ugc) = make_float2(g_done[0], g_done[1]);
+        at_bytes<float2>(d_dxo + o, ugc) = make_float2(g_done[0], g_done[1]);
         if (!DEFER) at_bytes<float2>(a.out2 + o, ugc) = make_float2(o_done[0], o_done[1]);
     };
     // Where the sources of the thread's two shell entries sit in the D window: read in FRONT of the
@@ -377,8 +458,9 @@ void chain_bwd(const ChainBwdArgs a) {
         hal[0] = tab(kTabHalo);
         hal[1] = tab(kTabHalo + 1);
     };
-    // behind a barrier that follows the element's last write of D
-    auto shell_of_done = [&](const unsigned (&hals)[2]) {
+    // behind a barrier that follows the element's last write of D; `n`: the iteration (ALL: the
+    // finished element is item n - 1, the one whose sums are complete item n - 2)
+    auto shell_of_done = [&](const unsigned (&hals)[2], int n) {
         const int hs = done_s;
         if (DEFER && hs >= 0) {
             // the thread's 18 shell weights sit side by side (stride 18 floats: nine conflict-free
@@ -391,7 +473,7 @@ void chain_bwd(const ChainBwdArgs a) {
                 hwv[2 * q + 1] = p2.y;
             }
             float t1 = t1_done, t2 = t2_done;
-            float *rec = a.out2 + (long)hs * a.nblk * kShell;
+            float *rec = d_halo + (long)hs * a.nblk * kShell;
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
                 const unsigned hal = hals[e];
@@ -410,55 +492,174 @@ void chain_bwd(const ChainBwdArgs a) {
                     // store can still take it as a 32-bit lane offset beside the scalar base
                     unsigned off = tab(kTabDst + e);
                     asm volatile("" : "+v"(off));
-                    at_bytes<float>(rec, off) = acc;
+                    if (ALL) st_agent(&at_bytes<float>(rec, off), acc);
+                    else at_bytes<float>(rec, off) = acc;
                 }
             }
             t1 = slot_wave_sum<256>(t1);
             t2 = slot_wave_sum<256>(t2);
+            // the two halves of `red` alternate by element; ALL: by iteration (a step may have an odd
+            // number of elements)
             if ((tid & 63) == 0)
-                *reinterpret_cast<float2 *>(red + (hs & 1) * 8 + 2 * (tid >> 6)) = make_float2(t1, t2);
+                *reinterpret_cast<float2 *>(red + ((ALL ? n + 1 : hs) & 1) * 8 + 2 * (tid >> 6)) = make_float2(t1, t2);
         }
         // the sums of the element before that one: its four waves' shares, in a fixed order (they
         // were written a barrier ago, into the other half of `red`)
-        if (DEFER && sums_s >= 0 && tid == 0) {
-            const float *r = red + (sums_s & 1) * 8;
+        if (DEFER && sums_s >= 0 && tid == 0 && (!ALL || n - 2 < counted)) {
+            const float *r = red + ((ALL ? n : sums_s) & 1) * 8;
             float *to = a.x_part + ((long)sums_s * a.nblk + blk) * 2;
-            to[0] = (r[0] + r[2]) + (r[4] + r[6]);
-            to[1] = (r[1] + r[3]) + (r[5] + r[7]);
+            const float p0 = (r[0] + r[2]) + (r[4] + r[6]), p1 = (r[1] + r[3]) + (r[5] + r[7]);
+            if (ALL) {
+                st_agent(to, p0);
+                st_agent(to + 1, p1);
+            } else {
+                to[0] = p0;
+                to[1] = p1;
+            }
         }
         sums_s = hs;
         done_s = -1;
     };
 
     if (ln_in) lds_barrier();  // the packed gamma and beta
-    if (s0 < s1) {
-        fetch_window(s0);
+    // ALL: `ready_word` is the ready word of the item at hand's counterpart in the step after
+    // (item n - B), requested while the element before was worked on.  `duty` is the next item this
+    // workgroup is in charge of (blk, blk + nblk, ...), `duty_count` what its counter read an
+    // iteration ago (0: not asked yet).
+    int j = ALL ? a.steps - 1 : 0, s = s0;
+    unsigned ready_word = 1u, duty_count = 0u;
+    int duty = blk;
+    bool gave_up = false;
+    // The workgroup in charge of item m (element fs of its step), once every block has counted
+    // itself in: the blocks' shares become the two means of the LayerNorm backward in front of that
+    // step (wave 0, block order, in double: always the same bits) -- the sums that item m + B will
+    // ask for -- and, once those are in memory, the item's ready word is set.
+    auto finalize = [&](int m) {
+        const int fs = m % a.B;
+        const float *part = a.x_part + (long)fs * a.nblk * 2;
+        double t1 = 0.0, t2 = 0.0;
+        for (int i0 = 0; i0 < a.nblk; i0 += 512) {
+            float2 v[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) v[q] = ld_agent2(part + 2 * min(i0 + q * 64 + tid, a.nblk - 1));
+#pragma unroll
+            for (int q = 0; q < 8; ++q)
+                if (i0 + q * 64 + tid < a.nblk) {
+                    t1 += (double)v[q].x;
+                    t2 += (double)v[q].y;
+                }
+        }
+        t1 = wave_sum(t1);
+        t2 = wave_sum(t2);
+        if (tid == 0) {
+            float *to = a.sums + 2 * (long)(m + a.B);
+            st_agent(to, (float)(t1 / (double)cells));
+            st_agent(to + 1, (float)(t2 / (double)cells));
+        }
+        wait_global_loads();  // ... and stores: the two means have been acknowledged
+        if (tid == 0 && a.spin_limit >= 0) st_agent(a.ready + m, 1u);
+    };
+    // Wave 0: the item in charge of is complete when its counter reads the number of blocks.
+    auto do_duty = [&](unsigned count) {
+        if (duty < counted && __builtin_amdgcn_readfirstlane(count) == (unsigned)a.nblk) {
+            finalize(duty);
+            duty += a.nblk;
+        }
+    };
+    // A bounded wait for a ready word (one wave; the loop runs on the scalar unit).  Wave 0 keeps
+    // looking after the item it is in charge of meanwhile: the word it waits for may be that very one.
+    auto wait_ready = [&](const unsigned *word, unsigned seen) {
+        unsigned v = __builtin_amdgcn_readfirstlane(seen);
+        const int limit = a.spin_limit < 0 ? -a.spin_limit : a.spin_limit;
+        int spins = 0;
+        while (v == 0u && !gave_up) {
+            __builtin_amdgcn_s_sleep(16);
+            if (tid < 64 && duty < counted) do_duty(ld_agent_uniform(a.arrive + duty));
+            v = __builtin_amdgcn_readfirstlane(ld_agent_uniform(word));
+            if (v == 0u && (++spins > limit || __builtin_amdgcn_readfirstlane(ld_agent_uniform(a.status)) != 0u)) {
+                gave_up = true;
+                if ((tid & 63) == 0) st_agent(a.status, 1u);
+            }
+        }
+    };
+    if (ALL) enter_step(j);
+    if (items > 0) {
+        fetch_window(c_x, c_xst, c_ln, s0);
         commit_window();
     }
-    for (int s = s0; s < s1; ++s) {
-        take_turns(s);
+    for (int n = 0; n < items; ++n) {
+        take_turns(ALL ? n : s);
+        if (ALL) {
+            // the walk's counters are the same for every lane; said here, where the loop's joins
+            // (one wave finalizes, one thread counts in) would otherwise make the compiler keep
+            // them, and every address built on them, in vector registers
+            j = __builtin_amdgcn_readfirstlane(j);
+            s = __builtin_amdgcn_readfirstlane(s);
+            // Everything this wave has stored so far was issued an iteration ago or earlier; once it
+            // is acknowledged, the barrier below lets thread 0 count the workgroup in for the item
+            // those stores complete.
+            wait_global_loads();
+            if (tid < 64) do_duty(duty_count);
+            if (n >= a.B) wait_ready(a.ready + (n - a.B), ready_word);
+        }
         // Requests first, stores behind them: loads and stores retire through one in-order
         // counter, and no wait for a load may include the stores.  This element's gradient (used
         // after the recompute, which hides the trip), then the next element's window.  All of it
         // in front of the barrier: none of it touches the windows, and the wait for the other
         // waves covers the issue.
         const long at = (long)s * cells;
-        const float2 dy2 = at_bytes<float2>(a.dy + at, ugc), yr2 = at_bytes<float2>(a.y_raw + at, ugc);
-        const float *rec = hin + ((long)s * a.nblk + blk) * kShell;
+        // ALL: with a later step, its workgroups left this element's gradient (this workgroup its
+        // own cells' part, the neighbours the rest)
+        const bool ei = ALL ? c_later && ei0 : ei0, ej = ALL ? c_later && ej0 : ej0, ek = ALL ? c_later && ek0 : ek0;
+        const float2 dy2 = at_bytes<float2>(c_dy + at, ugc), yr2 = at_bytes<float2>(c_yr + at, ugc);
+        const float *rec = c_rec + ((long)s * a.nblk + blk) * kShell;
         const unsigned oa = tab(kTabIn), ob = tab(kTabIn + 1), oc = tab(kTabIn + 2);
         auto off10 = [](unsigned word, int k) { return 4u * ((word >> (10 * k)) & 1023u); };
-        const float2 in_i = at_bytes<float2>(rec, off10(oa, 0)), in_j = at_bytes<float2>(rec, off10(oa, 1)),
-                     in_ij = at_bytes<float2>(rec, off10(oa, 2));
-        const float in_k = at_bytes<float>(rec, off10(ob, 0)), in_ik = at_bytes<float>(rec, off10(ob, 1)),
-                    in_jk = at_bytes<float>(rec, off10(ob, 2)), in_c = at_bytes<float>(rec, off10(oc, 0));
-        const float ny0 = load_ahead(a.y_stats, 2 * s), ny1 = load_ahead(a.y_stats, 2 * s + 1),
-                    ny2 = load_ahead(a.y_sums, 2 * s), ny3 = load_ahead(a.y_sums, 2 * s + 1);
-        fetch_window(min(s + 1, s1 - 1));
+        constexpr bool COH = ALL;
+        auto in2 = [&](unsigned off) { return COH ? ld_agent2(&at_bytes<float>(rec, off)) : at_bytes<float2>(rec, off); };
+        auto in1 = [&](unsigned off) { return COH ? ld_agent(&at_bytes<float>(rec, off)) : at_bytes<float>(rec, off); };
+        const float2 in_i = in2(off10(oa, 0)), in_j = in2(off10(oa, 1)), in_ij = in2(off10(oa, 2));
+        const float in_k = in1(off10(ob, 0)), in_ik = in1(off10(ob, 1)), in_jk = in1(off10(ob, 2)),
+                    in_c = in1(off10(oc, 0));
+        const float ny0 = load_ahead(c_ystat, 2 * s), ny1 = load_ahead(c_ystat, 2 * s + 1),
+                    ny2 = ALL ? ld_agent_uniform(a.sums + 2 * n) : load_ahead(a.y_sums, 2 * s),
+                    ny3 = ALL ? ld_agent_uniform(a.sums + 2 * n + 1) : load_ahead(a.y_sums, 2 * s + 1);
+        // the element after this one: the next of the step, or the first of the step before
+        int s2 = ALL ? s + 1 : min(s + 1, s1 - 1);
+        bool wrap = false;
+        if (ALL) {
+            if (n + 1 == items) s2 = s;
+            else if (s2 == a.B) {
+                s2 = 0;
+                wrap = true;
+            }
+        }
+        if (ALL && wrap) {  // once per step
+            const bool ln2 = j > 1;
+            fetch_window(ln2 ? a.y_raw + (j - 2) * a.step_floats : a.x0, a.y_stats + (long)(ln2 ? j - 2 : 0) * 2 * a.B,
+                         ln2, 0);
+        } else {
+            fetch_window(c_x, c_xst, c_ln, s2);
+        }
+        if (ALL) {
+            ready_word = (n + 1 >= a.B && n + 1 < items) ? ld_agent_uniform(a.ready + (n + 1 - a.B)) : 1u;
+            // the item in charge of: this workgroup itself counts in for item m in iteration m + 3
+            duty_count = (tid < 64 && duty < counted && duty + 3 <= n) ? ld_agent_uniform(a.arrive + duty) : 0u;
+        }
         store_done();
         unsigned shc[2];
         shell_sources(shc);
         lds_barrier();  // this element's window is in place; the last round's LDS readers are done
-        shell_of_done(shc);
+        if (ALL && n >= 3 && n - 3 < counted) {
+            // Item n - 3 is counted in: every wave has seen its stores for it acknowledged (halo
+            // values two iterations ago, the LayerNorm shares one), and the barrier has gathered the
+            // waves.  (This file is compiled with the compiler's rewrite of uniform atomics switched
+            // off: it turns the add into a wave-wide reduction with a returned count that it waits
+            // for at once, and with it for every request issued above.)
+            if (tid == 0)
+                (void)__hip_atomic_fetch_add(a.arrive + (n - 3), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        shell_of_done(shc, n);
 
         // ---- forward recompute; u_i of the owned cells is remembered ----
         float xcur[CPT];
@@ -574,18 +775,24 @@ void chain_bwd(const ChainBwdArgs a) {
             for (int c = 0; c < CPT; ++c) o_done[c] = dsum[c];
         }
         done_s = s;
+        if (ALL) {
+            d_dxo = c_dxo;
+            d_halo = c_halo;
+        }
 #pragma unroll
         for (int c = 0; c < CPT; ++c) g_done[c] = g[c];
         // the x windows are free (nothing reads them after the last barrier of the sweep)
-        if (s + 1 < s1) commit_window();
+        if (n + 1 < items) commit_window();
+        if (ALL && wrap) enter_step(--j);
+        s = ALL ? s2 : s + 1;
     }
     store_done();
     unsigned shc[2];
     shell_sources(shc);
     lds_barrier();  // the last element's D
-    shell_of_done(shc);
+    shell_of_done(shc, items);
     lds_barrier();  // its sums
-    shell_of_done(shc);
+    shell_of_done(shc, items + 1);
 
     // ---- parameter gradients ----
     const long slab_off = slab_offset();
@@ -682,6 +889,113 @@ template <int ACT, bool DEFER> int launch_chain(const StepArgs &a, hipStream_t s
     return step_cross_launch(a, k.nchunk, k.chunk_len, st);
 }
 
+// What the last step of a one-launch chain leaves in its records is added to dx here: the
+// chain's input gradient is wanted finished.  Same adds in the same order as chain_bwd makes
+// them for the steps inside the chain.
+__global__ __launch_bounds__(256) void chain_halo_gather(float *__restrict__ dx, const float *__restrict__ halo,
+                                                         int M, int N, int K, int nblk) {
+    using TL = ChainTile;
+    constexpr int BS = 8, CPT = 2;
+    const int blk = blockIdx.x, s = blockIdx.y, tid = threadIdx.x;
+    const Place<TL, CPT, 1> pl(tid, blk, N, K);
+    const int kb = K / BS, nb = N / BS, mb = M / BS;
+    const int bi = blk / (kb * nb), bj = (blk / kb) % nb, bk = blk % kb;
+    const int fi = pl.i == 0 ? 0 : pl.i == BS - 1 ? 1 : -1, fj = pl.j == 0 ? 0 : pl.j == BS - 1 ? 1 : -1,
+              fk = pl.kt == 0 ? 0 : pl.kt == TL::KT - 1 ? 1 : -1;
+    const bool ei = fi == 0 ? bi > 0 : fi == 1 ? bi < mb - 1 : false;
+    const bool ej = fj == 0 ? bj > 0 : fj == 1 ? bj < nb - 1 : false;
+    const bool ek = fk == 0 ? bk > 0 : fk == 1 ? bk < kb - 1 : false;
+    if (!(ei || ej || ek)) return;
+    const int zi = max(fi, 0), zj = max(fj, 0), zk = max(fk, 0), k2 = pl.kt * CPT;
+    const float *rec = halo + ((long)s * nblk + blk) * kShell;
+    float2 *at = reinterpret_cast<float2 *>(dx + (long)s * M * N * K + pl.gc);
+    float2 tot = *at;
+    auto pair_at = [&](int off) { return *reinterpret_cast<const float2 *>(rec + off); };
+    if (ei) { const float2 v = pair_at(kSegI + zi * 64 + pl.j * 8 + k2); tot.x += v.x; tot.y += v.y; }
+    if (ej) { const float2 v = pair_at(kSegJ + zj * 64 + pl.i * 8 + k2); tot.x += v.x; tot.y += v.y; }
+    if (ei && ej) { const float2 v = pair_at(kSegIJ + (zi * 2 + zj) * 8 + k2); tot.x += v.x; tot.y += v.y; }
+    float ends = 0.f;
+    if (ek) ends += rec[kSegK + zk * 64 + pl.i * 8 + pl.j];
+    if (ei && ek) ends += rec[kSegIK + (zi * 2 + zk) * 8 + pl.j];
+    if (ej && ek) ends += rec[kSegJK + (zj * 2 + zk) * 8 + pl.i];
+    if (ei && ej && ek) ends += rec[kSegC + zi * 4 + zj * 2 + zk];
+    tot.x += fk == 0 ? ends : 0.f;
+    tot.y += fk == 1 ? ends : 0.f;
+    *at = tot;
+}
+
+// ---- the whole chain in one launch -----------------------------------------------------------
+// workspace: [status word, counters, ready words | LayerNorm sums by item | LayerNorm shares of the
+// blocks | two halo buffers | the second dx buffer | scratch of the last LayerNorm's sums]
+struct ChainAllLayout {
+    size_t sync_words, sums_at, part_at, halo_at, halo_floats, dx_at, ln_at, total;
+};
+ChainAllLayout chain_all_layout(const ChainAll &c) {
+    auto up = [](size_t v) { return (v + 255) / 256 * 256; };
+    const size_t cells = (size_t)c.M * c.N * c.K, nblk = cells / 512;
+    ChainAllLayout l{};
+    l.sync_words = 64 + 2 * (size_t)c.outer * c.B;
+    l.sums_at = up(l.sync_words * 4);
+    l.part_at = up(l.sums_at + (size_t)c.outer * c.B * 2 * 4);
+    l.halo_at = up(l.part_at + (size_t)c.B * nblk * 2 * 4);
+    l.halo_floats = (size_t)c.B * nblk * kShell;
+    l.dx_at = up(l.halo_at + 2 * l.halo_floats * 4);
+    l.ln_at = up(l.dx_at + (size_t)c.B * cells * 4);
+    l.total = l.ln_at + layernorm_workspace(GRIDNET_F32, c.B, (long)cells);
+    return l;
+}
+
+template <int ACT> int launch_chain_all(const ChainAll &c, hipStream_t st) {
+    auto kern = chain_bwd<ACT, true, true>;
+    const size_t lds = (size_t)chain_lds_floats(c.inner) * sizeof(float);
+    static bool big_lds_enabled = false;
+    if (lds > 64 * 1024 && !big_lds_enabled) {
+        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           (int)((size_t)chain_lds_floats(kChainMaxInner) * sizeof(float)));
+        if (e != hipSuccess)
+            return fail(GRIDNET_ERR_LAUNCH, "cannot enable %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+        big_lds_enabled = true;
+    }
+    const long cells = (long)c.M * c.N * c.K;
+    const ChainAllLayout l = chain_all_layout(c);
+    char *ws = (char *)c.workspace;
+    ChainBwdArgs k{};
+    k.nblk = (int)(cells / 512);
+    k.nchunk = 1;
+    k.chunk_len = c.B;
+    k.param_mode = (c.flags & GRIDNET_OVERWRITE_PARAMS) ? kParamStore : kParamAddExclusive;
+    k.weight = c.weight; k.bias = c.bias; k.scale = c.scale; k.gamma = c.gamma; k.beta = c.beta;
+    k.x0 = c.x0; k.y_raw = c.y_raw; k.y_stats = c.stats; k.sums = (float *)(ws + l.sums_at); k.dy = c.dy;
+    k.dweight = c.dweight; k.dbias = c.dbias; k.dscale = c.dscale; k.dgamma = c.dgamma; k.dbeta = c.dbeta;
+    k.x_part = (float *)(ws + l.part_at);
+    k.halo_even = (float *)(ws + l.halo_at);
+    k.halo_odd = k.halo_even + l.halo_floats;
+    k.dx_even = c.dx;
+    k.dx_odd = (float *)(ws + l.dx_at);
+    k.status = (unsigned *)ws;
+    k.arrive = k.status + 64;
+    k.ready = k.arrive + (size_t)c.outer * c.B;  // (the last step's share of either array stays unused)
+    k.steps = c.outer;
+    k.spin_limit = c.spin_limit;
+    k.step_floats = (long)c.B * cells;
+    k.B = c.B; k.M = c.M; k.N = c.N; k.K = c.K; k.inner = c.inner;
+    // the sums of the last LayerNorm come from the gradient handed in
+    const long last = c.outer - 1;
+    if (int rc = layernorm_backward_sums(c.dy, c.y_raw + last * k.step_floats, c.stats + last * 2 * c.B, c.gamma,
+                                         k.sums, c.B, cells, (float *)(ws + l.ln_at), st))
+        return rc;
+    if (int rc = plan_fill_zero((float *)ws, (long)l.sync_words, st)) return rc;
+    void *args[] = {&k};
+    hipError_t e = hipLaunchCooperativeKernel((const void *)kern, dim3(padded_grid(k.nblk, 1)), dim3(256), args,
+                                              (unsigned)lds, st);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(GRIDNET_ERR_LAUNCH, "chain_bwd (whole chain): cooperative launch failed: %s", hipGetErrorString(e));
+    }
+    hipLaunchKernelGGL(chain_halo_gather, dim3(k.nblk, c.B), dim3(256), 0, st, c.dx, k.halo_even, c.M, c.N, c.K, k.nblk);
+    return check_launch("chain_halo_gather");
+}
+
 template <int ACT> int dispatch_defer(const StepArgs &a, hipStream_t st) {
     return a.ln.halo_out ? launch_chain<ACT, true>(a, st) : launch_chain<ACT, false>(a, st);
 }
@@ -695,6 +1009,44 @@ bool chain_supports(const StepArgs &a) {
 
 size_t chain_halo_floats(const StepArgs &a) {
     return (size_t)a.B * (a.M / 8) * (a.N / 8) * (a.K / 8) * kShell;
+}
+
+// The whole chain fits one launch when every block gets a workgroup of its own and all of them
+// are resident at once; a pair (step, element) must have been counted in and finalized (four
+// iterations after it was worked on) before the same workgroup can need it (B iterations after).
+constexpr int kChainAllMinBatch = 6;
+bool chain_all_supports(int B, int M, int N, int K, int inner, int outer) {
+    if (M <= 0 || N <= 0 || K <= 0 || M % 8 || N % 8 || K % 8) return false;
+    if (inner < 1 || inner > kChainMaxInner || outer < 2 || B < kChainAllMinBatch) return false;
+    if ((long)M * N * K * 27 >= (1L << 31)) return false;
+    static int per_cu_cache[kChainMaxInner + 1];
+    int &per_cu = per_cu_cache[inner];
+    if (per_cu == 0) {
+        auto kern = chain_bwd<GRIDNET_ACT_LEAKY_RELU, true, true>;
+        const size_t lds = (size_t)chain_lds_floats(inner) * sizeof(float);
+        if (lds > 64 * 1024 &&
+            hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)((size_t)chain_lds_floats(kChainMaxInner) * sizeof(float))) != hipSuccess)
+            return false;
+        int n = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, 256, lds) != hipSuccess || n < 1) n = -1;
+        per_cu = n;
+    }
+    if (per_cu < 1) return false;
+    const long nblk = (long)(M / 8) * (N / 8) * (K / 8);
+    return padded_grid((int)nblk, 1) <= (long)per_cu * plan_device_cus();
+}
+
+size_t chain_all_workspace(const ChainAll &c) { return chain_all_layout(c).total; }
+
+int chain_backward_all(const ChainAll &c, hipStream_t st) {
+    switch (c.activation) {
+        case GRIDNET_ACT_RELU: return launch_chain_all<GRIDNET_ACT_RELU>(c, st);
+        case GRIDNET_ACT_LEAKY_RELU: return launch_chain_all<GRIDNET_ACT_LEAKY_RELU>(c, st);
+        case GRIDNET_ACT_SILU: return launch_chain_all<GRIDNET_ACT_SILU>(c, st);
+        case GRIDNET_ACT_TANH: return launch_chain_all<GRIDNET_ACT_TANH>(c, st);
+    }
+    return fail(GRIDNET_ERR_ACTIVATION, "unknown activation function: id %d", c.activation);
 }
 
 int chain_backward(const StepArgs &a, hipStream_t st) {

@@ -113,6 +113,25 @@ bool chain_supports(const StepArgs &a);
 size_t chain_halo_floats(const StepArgs &a);
 int chain_backward(const StepArgs &a, hipStream_t st);
 
+// chain_bwd.hip: the backward of a whole chain of `outer` steps (one parameter set) in ONE launch
+// of resident workgroups that hand the cross-block values and the LayerNorm sums from step to
+// step through memory behind per-(step, element) counters.  y_raw [outer,B,M,N,K], stats
+// [outer,B,2]; dx receives the gradient of the chain's input x0.  The first word of the
+// workspace is a status: non-zero after the launch means a bounded wait ran out and the results
+// are invalid.
+struct ChainAll {
+    const float *weight, *bias, *scale, *gamma, *beta;
+    const float *x0, *y_raw, *stats, *dy;
+    float *dweight, *dbias, *dscale, *dgamma, *dbeta, *dx;
+    int B, M, N, K, inner, outer, activation, flags;
+    void *workspace;
+    size_t workspace_bytes;
+    int spin_limit;  // polls before a wait gives up; negative: ready words are never set (tests of the give-up path)
+};
+bool chain_all_supports(int B, int M, int N, int K, int inner, int outer);
+size_t chain_all_workspace(const ChainAll &c);
+int chain_backward_all(const ChainAll &c, hipStream_t st);
+
 // step_fast.hip: the cross-block kernel on two weight sets, for gated_fast.hip
 int gated_cross_launch(const StepArgs &a, const float *dsum, int nchunk, int chunk_len, hipStream_t st);
 

@@ -46,6 +46,10 @@ EXPORTS = (
     "gridnet_hip_chain_supported",
     "gridnet_hip_chain_halo_floats",
     "gridnet_hip_chain_backward",
+    "gridnet_hip_chain_all_supported",
+    "gridnet_hip_chain_all_workspace_bytes",
+    "gridnet_hip_chain_backward_all",
+    "gridnet_hip_chain_set_spin_limit",
     "gridnet_hip_probe",
 )
 
@@ -111,6 +115,14 @@ def _load():
     lib.gridnet_hip_chain_halo_floats.argtypes = [i, i, i, i, i]
     lib.gridnet_hip_chain_backward.restype = i
     lib.gridnet_hip_chain_backward.argtypes = [i] + [p] * 20 + [i] * 8 + [p, z, p]
+    lib.gridnet_hip_chain_all_supported.restype = i
+    lib.gridnet_hip_chain_all_supported.argtypes = [i] * 9
+    lib.gridnet_hip_chain_all_workspace_bytes.restype = z
+    lib.gridnet_hip_chain_all_workspace_bytes.argtypes = [i] * 7
+    lib.gridnet_hip_chain_backward_all.restype = i
+    lib.gridnet_hip_chain_backward_all.argtypes = [i] + [p] * 15 + [i] * 9 + [p, z, p]
+    lib.gridnet_hip_chain_set_spin_limit.restype = i
+    lib.gridnet_hip_chain_set_spin_limit.argtypes = [i]
     lib.gridnet_hip_probe.restype = i
     lib.gridnet_hip_probe.argtypes = [i, ctypes.POINTER(ctypes.c_double)]
     return lib

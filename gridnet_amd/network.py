@@ -56,7 +56,9 @@ class FusedBodyOp(torch.autograd.Function):
             raise RuntimeError("FusedBodyOp: the buffers of this forward were released by its first "
                                "backward; a second backward (retain_graph=True) is not supported")
         ctx.saved_tensors  # raises if an input was modified in place since the forward
-        dw, db, dr, dgamma, dbeta, dx0 = run.backward(grad_out.contiguous())
+        # checked: the one-launch chain backward reports through a status word whether its bounded
+        # waits held (read after a synchronisation; a failed launch is repeated step by step)
+        dw, db, dr, dgamma, dbeta, dx0 = run.backward_checked(grad_out.contiguous())
         if ctx.separate:
             grads = [g for triple in zip(dw, db, dr) for g in triple]
         else:

@@ -16,6 +16,14 @@ backward of a chain goes through ``gridnet_hip_chain_backward``
 step instead of finishing every dx (one kernel per step instead of two).  Same results to
 rounding.
 
+Where the whole grid fits the GPU at once (every block a resident workgroup: a 64^3 grid on an
+MI355X) and the steps share one parameter set, the chain backward is ONE launch
+(``gridnet_hip_chain_backward_all``, ``chain_all=None`` picks it when the grid fills the chip,
+``True`` wherever the library supports it, ``False`` never): the workgroups keep their blocks,
+weights and gradient accumulators from step to step and signal each other through memory.  Its
+waits are bounded; ``chain_all_status()`` (which synchronises) tells whether one ran out, in which
+case ``backward`` must be repeated with ``chain_all`` off -- ``backward_checked`` does both.
+
 ``weight``, ``bias`` and ``scale`` may each be a list of ``outer`` tensors: one parameter set
 per outer step (the reference's ``--separate_params``, gridnet/scripts/train_imagenet.py:54-58).
 ``backward`` then returns lists of gradients for them, one entry per step.
@@ -34,7 +42,8 @@ class BodyRunner:
     def __init__(self, weight, bias, scale, gamma, beta, batch: int, inner: int, outer: int,
                  block_size: int, activation: str = "leaky_relu", normalize: bool = False,
                  eps: float = 1e-5, ln_eps: float = 1e-5, backward: bool = True,
-                 fused: bool = False, outer_residual: bool = False, chain: bool = True):
+                 fused: bool = False, outer_residual: bool = False, chain: bool = True,
+                 chain_all=None):
         self.separate = isinstance(weight, (list, tuple))
         if self.separate:
             if not (len(weight) == len(bias) == len(scale) == outer):
@@ -68,7 +77,9 @@ class BodyRunner:
         if fused and outer_residual:
             n_s = 2 if backward else 1
         self.h = [torch.empty(shape, device=dev, dtype=dtype) for _ in range(n_h)]
-        self.s = [torch.empty(shape, device=dev, dtype=dtype) for _ in range(n_s)]
+        # one allocation: the one-launch chain backward takes the raw outputs as [outer, B, M, N, K]
+        self.s_all = torch.empty((n_s,) + shape, device=dev, dtype=dtype)
+        self.s = list(self.s_all)
         self.mean = torch.empty(keep, batch, device=dev, dtype=dtype)
         self.rstd = torch.empty(keep, batch, device=dev, dtype=dtype)
         self.ln_ws_bytes = _n.lib.gridnet_hip_layernorm_workspace_bytes(self.dt, batch, n)
@@ -115,6 +126,17 @@ class BodyRunner:
             # values over in
             nfl = _n.lib.gridnet_hip_chain_halo_floats(batch, self.M, self.N, self.K, block_size)
             self.halo = [torch.empty(nfl, device=dev, dtype=dtype) for _ in range(2 if outer > 1 else 0)]
+        self.chain_all = False
+        if self.chain and not self.separate and chain_all is not False and \
+                _n.lib.gridnet_hip_chain_all_supported(self.dt, batch, self.M, self.N, self.K, inner, outer,
+                                                       block_size, self.normalize):
+            nblk = (self.M // 8) * (self.N // 8) * (self.K // 8)
+            cus = torch.cuda.get_device_properties(dev).multi_processor_count
+            self.chain_all = bool(chain_all) or nblk >= cus
+        if self.chain_all:
+            self.ca_ws_bytes = _n.lib.gridnet_hip_chain_all_workspace_bytes(
+                batch, self.M, self.N, self.K, inner, outer, block_size)
+            self.ca_ws = _n.workspace(self.ca_ws_bytes, dev)
 
     def _params(self, j):
         """Device pointers of the parameter set of outer step j."""
@@ -248,7 +270,37 @@ class BodyRunner:
         torch.add(dn[1], grad_wrt(1), out=dn[1])
         return (*self._param_grads(), self.dgamma, self.dbeta, dn[1])
 
+    def chain_all_status(self) -> int:
+        """Synchronises.  Non-zero: a bounded wait of the last one-launch backward ran out and its
+        results are invalid."""
+        if not self.chain_all:
+            return 0
+        return int(self.ca_ws[:4].view(torch.int32).item())
+
+    def backward_checked(self, grad_out):
+        """``backward``; should the one-launch chain report that it gave up, the one-launch path is
+        switched off for this runner and the backward repeated launch by launch.  Synchronises."""
+        out = self.backward(grad_out)
+        if self.chain_all and self.chain_all_status() != 0:
+            self.chain_all = False
+            out = self.backward(grad_out)
+        return out
+
+    def _chain_all_backward(self, grad_out):
+        stream = _n.current_stream(self.w)
+        self._mark("step_bwd", 0)
+        _n.check(_n.lib.gridnet_hip_chain_backward_all(
+            self.dt, *self._params(0), self.gamma.data_ptr(), self.beta.data_ptr(), self.x0.data_ptr(),
+            self.s_all.data_ptr(), self.stats.data_ptr(), grad_out.data_ptr(),
+            *self._grads(0), self.dgamma.data_ptr(), self.dbeta.data_ptr(), self.ga.data_ptr(),
+            self.B, self.M, self.N, self.K, self.inner, self.outer, self.bs, self.act,
+            _n.OVERWRITE_PARAMS, self.ca_ws.data_ptr(), self.ca_ws_bytes, stream))
+        self._mark("step_bwd", 1)
+        return (*self._param_grads(), self.dgamma, self.dbeta, self.ga)
+
     def _fused_backward(self, grad_out):
+        if self.chain_all:
+            return self._chain_all_backward(grad_out)
         stream = _n.current_stream(self.w)
         last = self.outer - 1
         self._mark("ln_bwd", 0)

@@ -297,6 +297,47 @@ int gridnet_hip_chain_backward(int dtype, const void *weight, const void *bias, 
                                size_t workspace_bytes, void *stream);
 
 /*
+ * ---- The backward of a whole chain in one launch ------------------------------------------------
+ * The loop the reference's training scripts run around the step,
+ *     for i in range(outer): h = norm(net(h))          gridnet/scripts/train_imagenet.py:76-86
+ * (one Gridnet, one LayerNorm, shared by the steps), taken backward by ONE kernel whose workgroups
+ * stay resident for all `outer` steps: each keeps its block, its weights and its gradient
+ * accumulators from step to step and hands what crosses block boundaries, and the sums of the
+ * LayerNorm between two steps, to the workgroups that need them through memory, behind one
+ * counter per (step, batch element).  No set-up, drain or gradient read-modify-write per step.
+ *   x0      [B,M,N,K]        input of the chain
+ *   y_raw   [outer,B,M,N,K]  raw output of every step (gridnet_hip_fused_forward's y_raw)
+ *   stats   [outer,B,2]      their LayerNorm statistics (its y_stats)
+ *   dy      [B,M,N,K]        gradient with respect to LayerNorm(y_raw[outer-1])
+ *   dweight, dbias, dscale, dgamma, dbeta   accumulated, or written with GRIDNET_OVERWRITE_PARAMS
+ *   dx      [B,M,N,K]        gradient with respect to x0, fully written
+ * float32, normalize = false, block_size 8, 1 <= inner <= 4, outer >= 2, B >= 6, and a grid whose
+ * blocks all fit the GPU at once (M/8 * N/8 * K/8 workgroups resident: 512 on an MI355X, a 64^3
+ * grid); gridnet_hip_chain_all_supported() tells.  Results agree with the chain of
+ * gridnet_hip_chain_backward calls to rounding and are the same bits on every run.
+ * The kernel is launched cooperatively.  Every wait inside it is bounded: should one run out (the
+ * workgroups were not all resident after all), the kernel still ends, and the FIRST 4 BYTES OF THE
+ * WORKSPACE, zero otherwise, are non-zero once the stream has passed the call: the results are
+ * then invalid and the caller repeats the backward with gridnet_hip_chain_backward, whose inputs
+ * this call leaves untouched.
+ */
+int gridnet_hip_chain_all_supported(int dtype, int B, int M, int N, int K, int inner, int outer,
+                                    int block_size, int normalize);
+size_t gridnet_hip_chain_all_workspace_bytes(int B, int M, int N, int K, int inner, int outer,
+                                             int block_size);
+int gridnet_hip_chain_backward_all(int dtype, const void *weight, const void *bias, const void *scale,
+                                   const void *gamma, const void *beta, const void *x0,
+                                   const void *y_raw, const void *stats, const void *dy,
+                                   void *dweight, void *dbias, void *dscale, void *dgamma,
+                                   void *dbeta, void *dx, int B, int M, int N, int K, int inner,
+                                   int outer, int block_size, int activation, int flags,
+                                   void *workspace, size_t workspace_bytes, void *stream);
+/* How often a wait inside the one-launch chain kernels polls before it gives up (default 200000,
+ * about a second).  A negative value makes the kernels never signal completion to each other, so
+ * that every wait runs out after -limit polls: the give-up path, for tests.  Returns the old value. */
+int gridnet_hip_chain_set_spin_limit(int limit);
+
+/*
  * Machine ceilings, measured with the same compiler flags as the kernels, for a benchmark to
  * quote beside the vendor's peaks.  No counterpart in the reference and not part of the update
  * path.  Allocates and frees its own buffers, runs on the null stream and synchronises.
