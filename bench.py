@@ -110,6 +110,24 @@ def gpu_run(wl, steps, warmup, fused, graph_replay=True, chain_all=None):
     return wall, graph_s, kernel_s, bool(getattr(run, "chain_all", False))
 
 
+def what_binds(hbm_frac, valu_busy_pct, lds_busy_frac):
+    """One sentence from the figures of this line: which of HBM, vector ALU and LDS pipe the
+    dominant kernel keeps busiest, and whether that one is saturated."""
+    util = {"HBM bandwidth": hbm_frac,
+            "vector ALU": None if valu_busy_pct is None else valu_busy_pct / 100.0,
+            "LDS pipe": lds_busy_frac}
+    known = {k: v for k, v in util.items() if v is not None}
+    if not known:
+        return None
+    shown = ", ".join(f"{k} {100 * v:.0f} %" for k, v in known.items())
+    top = max(known, key=known.get)
+    if known[top] >= 0.8:
+        return f"{top} ({shown}; HBM against the vendor peak, the pipes as busy cycles from the profile)"
+    return (f"none of the three is saturated ({shown}; HBM against the vendor peak, the pipes as busy cycles "
+            f"from the profile): the busiest is the {top}, and the waves wait on LDS and ALU latency at the "
+            "occupancy the register file allows")
+
+
 def cpu_baseline(wl, budget_s=25.0):
     """The reference-style pure-torch path (block loop + gather; oracle.ref_style) composed with
     F.layer_norm, forward + autograd backward, on a bounded sample of the workload."""
@@ -204,7 +222,7 @@ def reference_benchmark_shape(steps, warmup):
     a, p = 2 * 32 ** 3 * 4, 32 ** 3 * 4
     algo = (2 * a + 29 * p) + (3 * a + 58 * p)  # one step forward, one step backward
     print(json.dumps({
-        "metric": "cell-updates/s fwd+bwd, 64^3 grid 8^3 blocks batch 32; % of HBM roofline",
+        "metric": "cell-updates/s fwd+bwd, reference benchmark shape 32^3 grid 8^3 blocks batch 2 inner 10 normalize",
         "value": cu / t_fb, "unit": "cell-updates/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": t_fb * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
@@ -255,11 +273,15 @@ def main():
     if fused:  # a fused entry point does the work of the step AND of the LayerNorm beside it
         bytes_["step_fwd"] += bytes_["ln_fwd"]
         bytes_["step_bwd"] += bytes_["ln_bwd"]
+    # the one-launch chain backward takes all outer steps in ONE call
+    steps_per_call = {"step_bwd": wl.outer} if one_launch else {}
+    for k, n_steps in steps_per_call.items():
+        bytes_[k] *= n_steps
     dominant = max(kernel_s, key=lambda k: kernel_s[k])
     # HBM bytes per call of that entry point and the counters of its main kernel, from the
     # committed rocprofv3 --pmc summaries (FETCH_SIZE and WRITE_SIZE scaled by a copy kernel of
     # known size); null if absent
-    traffic, counters, counted_kernel = None, {}, None
+    traffic, counters, counted_kernel, profile_source = None, {}, None, None
     try:
         with open(os.path.join(ROOT, "profiles", "counters.json")) as fh:
             variant = "normalize" if args.normalize else "fused" if fused else "steps"
@@ -267,19 +289,39 @@ def main():
             traffic = prof.get("traffic_bytes_per_call", {}).get(dominant)
             counted_kernel = prof.get("dominant_kernel", {}).get(dominant)
             counters = prof.get("kernels", {}).get(counted_kernel, {})
+            profile_source = prof.get("source")
     except OSError:
         pass
-    # ceilings of this machine, measured now by the library's probe kernels
-    from gridnet_amd import native
-    ceil = {k: native.probe(k) for k in native.PROBES}
-    lds_widths = {k: native.probe(k) for k in native.LDS_WIDTH_PROBES}
-    lds_peak = LDS_BYTES_PER_CLOCK_PER_CU * CUS * ceil["clock_ghz"]
+    # ceilings of this machine, measured now by the probe library (bench-only; a failure there
+    # must not cost the headline, so a figure that cannot be measured is reported as null)
+    import gc
+
+    import torch
+    gc.collect()
+    torch.cuda.empty_cache()  # the copy probe wants 2 GiB of its own
+    ceil, lds_widths = {}, {}
+    try:
+        from gridnet_amd import probe
+        for k in probe.PROBES:
+            try:
+                ceil[k] = probe.probe(k)
+            except RuntimeError as exc:
+                print(f"bench.py: probe {k} failed: {exc}", file=sys.stderr, flush=True)
+        for k in probe.LDS_WIDTH_PROBES:
+            try:
+                lds_widths[k] = probe.probe(k)
+            except RuntimeError as exc:
+                print(f"bench.py: probe {k} failed: {exc}", file=sys.stderr, flush=True)
+    except (ImportError, OSError) as exc:
+        print(f"bench.py: probe library unavailable: {exc}", file=sys.stderr, flush=True)
+    clock = ceil.get("clock_ghz")
+    lds_peak = None if clock is None else LDS_BYTES_PER_CLOCK_PER_CU * CUS * clock
     dom_s = kernel_s[dominant]
     achieved = bytes_[dominant] / dom_s / 1e9
     # the same entry point against the vector ALU: algorithmic fp32 FMAs per cell-update (27 for
     # the update itself; 81 in the backward: recompute, weight gradient, input gradient)
     fma = {"step_fwd": 27, "step_bwd": 81}.get(dominant)
-    per_launch = wl.cell_updates / wl.outer
+    per_launch = wl.cell_updates / wl.outer * steps_per_call.get(dominant, 1)
     tflops = None if fma is None else 2 * fma * per_launch / dom_s / 1e12
     out = {
         "metric": "cell-updates/s fwd+bwd, 64^3 grid 8^3 blocks batch 32; % of HBM roofline",
@@ -307,38 +349,38 @@ def main():
         "roofline": {
             "bound": "hbm",
             "kernel": dominant,
+            "outer_steps_per_call": steps_per_call.get(dominant, 1),
             "achieved": achieved,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
             "traffic": traffic,
+            "traffic_from_profile": profile_source,
         },
         # the same entry point against the vector ALU (fp32 FMAs without packed instructions) and
         # against the LDS pipes; the counter figures are those of the committed profile summary
         "vector_alu": {"kernel": dominant, "achieved": tflops, "unit": "TFLOP/s",
                        "peak": FP32_UNPACKED_PEAK_TFLOPS,
                        "frac": None if tflops is None else tflops / FP32_UNPACKED_PEAK_TFLOPS,
-                       "measured_fma_ceiling": 2 * ceil["fma_tfma_per_s"],
-                       "frac_of_measured_ceiling": None if tflops is None else tflops / (2 * ceil["fma_tfma_per_s"]),
+                       "measured_fma_ceiling": None if "fma_tfma_per_s" not in ceil else 2 * ceil["fma_tfma_per_s"],
+                       "frac_of_measured_ceiling": None if tflops is None or "fma_tfma_per_s" not in ceil
+                       else tflops / (2 * ceil["fma_tfma_per_s"]),
                        "valu_busy_pct": counters.get("valu_busy_pct"),
+                       "from_profile": profile_source,
                        "peak_with_packed_fp32": FP32_PEAK_TFLOPS},
-        "lds": {"kernel": counted_kernel, "unit": "GB/s",
+        "lds": {"kernel": counted_kernel, "unit": "GB/s", "from_profile": profile_source,
                 "achieved": counters.get("lds_gb_per_s_estimate"),
                 "peak": lds_peak,
-                "frac": None if not counters else counters["lds_gb_per_s_estimate"] / lds_peak,
+                "frac": None if not counters or not lds_peak else counters["lds_gb_per_s_estimate"] / lds_peak,
                 "busy_frac": counters.get("lds_busy_frac"),
                 "bank_conflict_frac_of_busy": counters.get("lds_conflict_frac_of_busy"),
-                "measured_read_ceiling": ceil["lds_gb_per_s"],
+                "measured_read_ceiling": ceil.get("lds_gb_per_s"),
                 "pipe_cycles_per_wave_read": lds_widths,
                 "peak_is": "128 B per clock and CU x 256 CUs x the measured core clock; 16-byte reads go "
                            "beyond it on this part, see measured_read_ceiling"},
-        "machine": {"core_clock_ghz_under_load": ceil["clock_ghz"],
-                    "hbm_copy_gb_per_s": ceil["copy_gb_per_s"]},
-        "binds": ("none of HBM, vector ALU and LDS is saturated by the dominant kernel: its waves wait on "
-                  "LDS and ALU latency at 2 waves per SIMD (the register file holds no more of them)")
-                 if wl.block_size == 8 else
-                 ("vector ALU and LDS pipes together (the busier of the two is above 70 % in both step "
-                  "kernels); HBM is far from its limit"),
+        "machine": {"core_clock_ghz_under_load": clock,
+                    "hbm_copy_gb_per_s": ceil.get("copy_gb_per_s")},
+        "binds": what_binds(achieved / HBM_PEAK_GBS, counters.get("valu_busy_pct"), counters.get("lds_busy_frac")),
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(wl)

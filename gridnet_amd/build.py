@@ -1,4 +1,5 @@
-"""Build recipe for libgridnet_hip.so (gfx950 only, hipcc, in-tree).
+"""Build recipe for libgridnet_hip.so and the benchmark's libgridnet_probe.so (gfx950 only, hipcc,
+in-tree).
 
 Usage: ``python -m gridnet_amd.build`` or ``gridnet_amd.build.build()``.
 """
@@ -11,7 +12,10 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libgridnet_hip.so")
-SOURCES = ["api.hip", "step_generic.hip", "step_fast.hip", "chain_bwd.hip", "gated_generic.hip", "gated_fast.hip", "layernorm.hip", "probe.hip"]
+SOURCES = ["api.hip", "step_generic.hip", "step_fast.hip", "chain_bwd.hip", "gated_generic.hip", "gated_fast.hip", "layernorm.hip"]
+# machine ceilings for bench.py: not part of the product library (it allocates and synchronises)
+PROBE_LIB = os.path.join(HERE, "libgridnet_probe.so")
+PROBE_SOURCES = ["probe.hip"]
 
 # -packed-fp32-ops is switched OFF on purpose: hipcc -O3 otherwise forms v_pk_*_f32 from
 # ordinary float code.
@@ -55,12 +59,15 @@ def build(verbose: bool = True, extra_flags=(), out=None, objdir=None) -> str:
             print(out)
         return obj
 
-    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
-        objs = list(pool.map(compile_one, SOURCES))
-    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", out]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.run(cmd, check=True)
+    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES) + len(PROBE_SOURCES))) as pool:
+        all_objs = list(pool.map(compile_one, SOURCES + PROBE_SOURCES))
+    objs, probe_objs = all_objs[:len(SOURCES)], all_objs[len(SOURCES):]
+    probe_out = os.path.join(os.path.dirname(out), os.path.basename(PROBE_LIB))
+    for target, members in ((out, objs), (probe_out, probe_objs)):
+        cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *members, "-o", target]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.run(cmd, check=True)
     return out
 
 

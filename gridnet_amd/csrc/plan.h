@@ -62,6 +62,10 @@ struct SlabTargets {
     int count;
 };
 
+// The slabs are 256-byte aligned and read as 16-byte vectors.  The caller's arrays are accessed as
+// 16-byte vectors too although the C ABI asks them to be aligned to their element size only:
+// gfx950 serves global accesses at any 4-byte alignment (a misaligned vector costs a second
+// request, nothing else); tests/test_gpu_alignment.py runs this with arrays 4 bytes off.
 __global__ void plan_reduce_slabs_f32(const float *slabs, int ncopies, long stride, SlabTargets t,
                                       long total4, int accumulate) {
     long i = (long)blockIdx.x * blockDim.x + threadIdx.x;

@@ -1,12 +1,40 @@
 // Machine ceilings measured with the library's own compiler flags, for the benchmark to quote
 // beside the vendor peaks: sustained unpacked fp32 FMA rate, LDS read rate, core clock under load
-// and a plain HBM copy.  Nothing on the update path calls these.
+// and an HBM copy.  A library of its own (libgridnet_probe.so) that only bench.py and its test
+// load: unlike libgridnet_hip.so it allocates, runs on the null stream and synchronises.
+//   gridnet_probe(what, &result): 0 on success
+//     0 FMA    sustained fp32 FMA rate without packed instructions, TFMA/s (x2 = TFLOP/s)
+//     1 LDS    conflict-free 16-byte LDS reads over all CUs, GB/s
+//     2 CLOCK  core clock while every CU runs the FMA loop, GHz
+//     3 COPY   device-to-device copy of 1 GiB, 16 bytes per lane, four requests in flight per
+//              lane, read + write GB/s
+//     4..7     cycles of one CU's LDS pipe per wave-level read instruction: 32-, 64-, 128-bit,
+//              and one two-address 64-bit read; lanes at consecutive addresses, 8 waves
+//   gridnet_probe_last_error(): message of the last failure on the calling thread
 #include <hip/hip_runtime.h>
 
-#include "common.h"
+#include <cstdarg>
+#include <cstdio>
 
 namespace gridnet {
 namespace {
+
+enum { GRIDNET_PROBE_FMA = 0, GRIDNET_PROBE_LDS = 1, GRIDNET_PROBE_CLOCK = 2, GRIDNET_PROBE_COPY = 3,
+       GRIDNET_PROBE_LDS_B32 = 4, GRIDNET_PROBE_LDS_B64 = 5, GRIDNET_PROBE_LDS_B128 = 6,
+       GRIDNET_PROBE_LDS_2XB64 = 7 };
+enum { GRIDNET_OK = 0, GRIDNET_ERR_ARGUMENT = 1, GRIDNET_ERR_LAUNCH = 5 };
+
+char *probe_error() {
+    static thread_local char buf[256] = {0};
+    return buf;
+}
+int fail(int status, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(probe_error(), 256, fmt, ap);
+    va_end(ap);
+    return status;
+}
 
 constexpr int kProbeThreads = 256;
 
@@ -106,10 +134,17 @@ __global__ __launch_bounds__(512) void probe_lds_width(float *out, long long *ti
     if (lane == 0) ticks[threadIdx.x / 64] = c1 - c0;
 }
 
+// 16 bytes per lane and request, four requests in flight per lane before the first store (n is a
+// multiple of 4 * the grid's threads)
 __global__ __launch_bounds__(kProbeThreads) void probe_copy(const float4 *src, float4 *dst, size_t n) {
-    size_t i = (size_t)blockIdx.x * kProbeThreads + threadIdx.x;
     const size_t stride = (size_t)gridDim.x * kProbeThreads;
-    for (; i < n; i += stride) dst[i] = src[i];
+    for (size_t i = (size_t)blockIdx.x * kProbeThreads + threadIdx.x; i + 3 * stride < n; i += 4 * stride) {
+        const float4 a = src[i], b = src[i + stride], c = src[i + 2 * stride], d = src[i + 3 * stride];
+        dst[i] = a;
+        dst[i + stride] = b;
+        dst[i + 2 * stride] = c;
+        dst[i + 3 * stride] = d;
+    }
 }
 
 struct Timer {
@@ -140,7 +175,9 @@ struct Timer {
 
 using namespace gridnet;
 
-extern "C" int gridnet_hip_probe(int what, double *result) {
+extern "C" const char *gridnet_probe_last_error(void) { return probe_error(); }
+
+extern "C" int gridnet_probe(int what, double *result) {
     if (!result) return fail(GRIDNET_ERR_ARGUMENT, "probe: result is null");
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess ||
@@ -186,8 +223,8 @@ extern "C" int gridnet_hip_probe(int what, double *result) {
             rc = fail(GRIDNET_ERR_LAUNCH, "probe: hipMalloc failed");
             break;
         }
-        hipLaunchKernelGGL(probe_copy, dim3(cus * 16), dim3(kProbeThreads), 0, 0, dst, src, n);  // first touch
-        s = timer.best(4, [&] { hipLaunchKernelGGL(probe_copy, dim3(cus * 16), dim3(kProbeThreads), 0, 0, src, dst, n); });
+        hipLaunchKernelGGL(probe_copy, dim3(cus * 32), dim3(kProbeThreads), 0, 0, dst, src, n);  // first touch
+        s = timer.best(4, [&] { hipLaunchKernelGGL(probe_copy, dim3(cus * 32), dim3(kProbeThreads), 0, 0, src, dst, n); });
         if (s > 0) *result = 2.0 * (double)n * sizeof(float4) / s / 1e9;
         break;
     }

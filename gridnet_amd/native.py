@@ -50,7 +50,6 @@ EXPORTS = (
     "gridnet_hip_chain_all_workspace_bytes",
     "gridnet_hip_chain_backward_all",
     "gridnet_hip_chain_set_spin_limit",
-    "gridnet_hip_probe",
 )
 
 
@@ -123,8 +122,6 @@ def _load():
     lib.gridnet_hip_chain_backward_all.argtypes = [i] + [p] * 15 + [i] * 9 + [p, z, p]
     lib.gridnet_hip_chain_set_spin_limit.restype = i
     lib.gridnet_hip_chain_set_spin_limit.argtypes = [i]
-    lib.gridnet_hip_probe.restype = i
-    lib.gridnet_hip_probe.argtypes = [i, ctypes.POINTER(ctypes.c_double)]
     return lib
 
 
@@ -132,19 +129,6 @@ try:
     lib = _load()
 except AttributeError as exc:  # an older build of the library without some entry point
     raise ImportError(f"{LIB_PATH} is stale ({exc}): rebuild with `python -m gridnet_amd.build`") from exc
-
-
-PROBES = {"fma_tfma_per_s": 0, "lds_gb_per_s": 1, "clock_ghz": 2, "copy_gb_per_s": 3}  # GRIDNET_PROBE_*
-# LDS-pipe cycles per wave-level read instruction, by width (GRIDNET_PROBE_LDS_B32 ... _2XB64)
-LDS_WIDTH_PROBES = {"ds_read_b32": 4, "ds_read_b64": 5, "ds_read_b128": 6, "ds_read2_b64": 7}
-
-
-def probe(what: str) -> float:
-    """One of the machine ceilings of gridnet_hip_probe on the current device."""
-    out = ctypes.c_double(0.0)
-    kind = PROBES[what] if what in PROBES else LDS_WIDTH_PROBES[what]
-    check(lib.gridnet_hip_probe(kind, ctypes.byref(out)))
-    return out.value
 
 
 def last_error() -> str:

@@ -115,9 +115,14 @@ int gridnet_hip_backward(int dtype, const void *weight, const void *bias, const 
  * code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.
  * The scratch that gridnet_hip_backward takes as `workspace` lives in a static device array of
  * GRIDNET_STATIC_SCRATCH_BYTES inside the library instead (one copy per GPU, held until the
- * process ends).  A problem that needs more (gridnet_hip_backward_workspace_bytes() tells) is
- * rejected with GRIDNET_ERR_WORKSPACE and nothing is enqueued.  Same arguments, results and
- * flags as gridnet_hip_backward otherwise (it runs the same kernels).
+ * process ends).  What must fit is the part gridnet_hip_backward cannot do without: B*M*N*K
+ * elements, plus two per (batch element, block) with normalize; a problem that needs more is
+ * rejected with GRIDNET_ERR_WORKSPACE and nothing is enqueued.  (The figure that
+ * gridnet_hip_backward_workspace_bytes() returns also counts, on grids with fewer blocks than
+ * compute units, room for one copy of the gradient arrays per batch chunk; with less of that
+ * room than gridnet_hip_backward was given the batch is split over fewer workgroups and the
+ * parameter gradients are summed in another order: equal to rounding, and still the same bits
+ * on every run.)  Same arguments and flags as gridnet_hip_backward, same kernels.
  * Every call on a GPU shares that GPU's array: calls that may overlap on one GPU (different
  * streams, different threads) race and must be serialised by the caller.  The array's
  * contents need not be, and are not, preserved between calls.
@@ -336,23 +341,6 @@ int gridnet_hip_chain_backward_all(int dtype, const void *weight, const void *bi
  * about a second).  A negative value makes the kernels never signal completion to each other, so
  * that every wait runs out after -limit polls: the give-up path, for tests.  Returns the old value. */
 int gridnet_hip_chain_set_spin_limit(int limit);
-
-/*
- * Machine ceilings, measured with the same compiler flags as the kernels, for a benchmark to
- * quote beside the vendor's peaks.  No counterpart in the reference and not part of the update
- * path.  Allocates and frees its own buffers, runs on the null stream and synchronises.
- *   GRIDNET_PROBE_FMA    sustained fp32 FMA rate without packed instructions, TFMA/s (x2 = TFLOP/s)
- *   GRIDNET_PROBE_LDS    conflict-free 16-byte LDS reads over all CUs, GB/s
- *   GRIDNET_PROBE_CLOCK  core clock while every CU runs the FMA loop, GHz
- *   GRIDNET_PROBE_COPY   device-to-device copy of 1 GiB by a plain kernel, read + write GB/s
- *   GRIDNET_PROBE_LDS_B32 / _B64 / _B128 / _2XB64   cycles of one CU's LDS pipe per wave-level read
- *                        instruction of that width (2XB64: one two-address 64-bit read), lanes at
- *                        consecutive addresses, 8 waves
- */
-enum { GRIDNET_PROBE_FMA = 0, GRIDNET_PROBE_LDS = 1, GRIDNET_PROBE_CLOCK = 2, GRIDNET_PROBE_COPY = 3,
-       GRIDNET_PROBE_LDS_B32 = 4, GRIDNET_PROBE_LDS_B64 = 5, GRIDNET_PROBE_LDS_B128 = 6,
-       GRIDNET_PROBE_LDS_2XB64 = 7 };
-int gridnet_hip_probe(int what, double *result);
 
 #ifdef __cplusplus
 }

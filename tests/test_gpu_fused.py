@@ -229,7 +229,9 @@ def test_fused_full_size_agrees_with_op_by_op_chain():
     ((8, 24, 16), 5, 2, 2, "tanh"),        # non-cubic, a single block along M (no neighbour there)
     ((24, 8, 8), 1, 3, 4, "silu"),         # one sample, blocks in a row
     ((16, 32, 24), 7, 4, 3, "silu"),
-    ((64, 64, 64), 2, 4, 3, "leaky_relu"), # 512 blocks: one workgroup per block, plain stores
+    ((64, 64, 64), 2, 4, 3, "silu"),       # 512 blocks: one workgroup per block, no gradient copies:
+                                           # plain stores on the last step, read-add-write on the others
+    ((64, 64, 64), 2, 4, 2, "leaky_relu"), # the same plan under the workloads' own activation (forward only)
     ((8, 8, 8), 4, 2, 3, "relu"),          # a single block: nothing crosses a boundary
     ((16, 16, 16), 2, 4, 1, "silu"),       # one outer step: the call that finishes dx itself
 ])
@@ -251,7 +253,7 @@ def test_chain_backward_matches_fused_backward(shape, batch, inner, outer, activ
     results = []
     for chain in (False, True):
         run = BodyRunner(*(v.to(DEV) for v in (w, b, r, gamma, beta)), batch, inner, outer, 8, activation,
-                         False, backward=True, fused=True, chain=chain)
+                         False, backward=True, fused=True, chain=chain, chain_all=False)
         assert run.chain == chain
         y = run.forward(x0.to(DEV)).clone()
         results.append((y, *[v.clone() for v in run.backward(gy.to(DEV))]))

@@ -247,22 +247,20 @@ def test_largest_grid_the_index_range_allows(bs):
 
 
 def test_machine_ceiling_probes_report_sane_figures():
-    """gridnet_hip_probe (the figures bench.py quotes beside the vendor peaks): every quantity comes
-    back positive and below what the part can do; an unknown quantity is refused."""
-    import ctypes
+    """libgridnet_probe.so (the figures bench.py quotes beside the vendor peaks; a library of its
+    own, not part of the update path): every quantity comes back positive and below what the part
+    can do; an unknown quantity is refused."""
+    from gridnet_amd import probe as p
 
-    from gridnet_amd import native as n
-
-    fma, lds, clock, copy = (n.probe(k) for k in ("fma_tfma_per_s", "lds_gb_per_s", "clock_ghz", "copy_gb_per_s"))
+    fma, lds, clock, copy = (p.probe(k) for k in ("fma_tfma_per_s", "lds_gb_per_s", "clock_ghz", "copy_gb_per_s"))
     print(f"probes: {fma:.1f} TFMA/s, LDS {lds:.0f} GB/s, {clock:.2f} GHz, copy {copy:.0f} GB/s", flush=True)
     assert 5.0 < fma < 80.0         # 39.3 TFMA/s is the unpacked fp32 peak of 256 CUs at 2.4 GHz
     assert 1.0e4 < lds < 4.0e5
     assert 0.5 < clock < 3.5
     assert 500.0 < copy < 8000.0    # read + write against 8 TB/s
-    widths = {k: n.probe(k) for k in n.LDS_WIDTH_PROBES}
+    widths = {k: p.probe(k) for k in p.LDS_WIDTH_PROBES}
     print("LDS pipe cycles per wave-level read:", {k: round(v, 2) for k, v in widths.items()}, flush=True)
     assert all(1.0 < v < 64.0 for v in widths.values())
     assert widths["ds_read_b32"] < widths["ds_read_b128"]
-    out = ctypes.c_double(0.0)
-    assert n.lib.gridnet_hip_probe(99, ctypes.byref(out)) != 0
-    assert "unknown" in n.last_error()
+    with pytest.raises(RuntimeError, match="unknown"):
+        p.probe_id(99)

@@ -73,6 +73,29 @@ def test_static_scratch_matches_workspace_entry_point_twice():
         assert torch.equal(a, b), f"{name}: static-scratch call differs from the workspace call"
 
 
+def test_static_scratch_call_matches_the_oracle():
+    """The same kernels run behind both entry points, so the comparison above checks the scratch
+    plumbing; this one holds a static-scratch call to the hand-derived backward of the oracle
+    (oracle/manual.py: the formulas of src/gridnet_cuda_kernels.cu:321-449 in fp64) at the bar."""
+    from gridnet_amd import native as n
+    from helpers import assert_close
+    from oracle.manual import gridnet_step_backward_manual
+
+    shape, batch, inner = (16, 16, 16), 3, 2
+    w, b, r = make_params(shape, seed=51)
+    x, gy = make_acts(batch, shape, seed=52), make_acts(batch, shape, seed=53)
+    d = [t.to(DEV) for t in (w, b, r, x, gy)]
+    outs = [torch.empty_like(t) for t in (d[0], d[1], d[2], d[3])]
+    n.check(n.lib.gridnet_hip_backward_static(
+        0, *[t.data_ptr() for t in d], *[o.data_ptr() for o in outs], batch, *shape, inner, 8, 1e-5, 0,
+        n.activation_id("silu"), n.OVERWRITE, n.current_stream(d[0])))
+    torch.cuda.synchronize()
+    dw, db, dr, dx = gridnet_step_backward_manual(w.double(), b.double(), r.double(), x.double(), gy.double(),
+                                                  inner, 8, 1e-5, False, "silu")
+    for name, got, exp in zip(("dweight", "dbias", "dscale", "dx"), outs, (dw, db, dr, dx)):
+        assert_close(got, exp, what=name)
+
+
 def test_static_scratch_rejects_what_does_not_fit():
     from gridnet_amd import native as n
 
