@@ -76,6 +76,9 @@ WORKLOADS = {
     "C4": Workload("C4 128^3 bs8 B8 inner4 outer16 fwd", 128, 8, 8, 4, 16, False, zero_bias=True,
                    embed="patches", classes=1000),
     "C5": Workload("C5 64^3 bs4 B128 inner8 outer16 fwd+bwd", 64, 4, 128, 8, 16, True),
+    # C3 with the inner iteration count of the reference's own ImageNet script
+    # (gridnet/scripts/train_imagenet.py:101-104: inner 8, outer 12, grid 64, batch 32)
+    "C3i8": Workload("C3i8 64^3 bs8 B32 inner8 outer12 fwd+bwd", 64, 8, 32, 8, 12, True),
 }
 
 

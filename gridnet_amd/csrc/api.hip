@@ -540,7 +540,7 @@ int gridnet_hip_chain_backward(int dtype, const void *weight, const void *bias, 
     a.ln.gamma = (const float *)gamma;
     if (!chain_supports(a))
         return fail(GRIDNET_ERR_ARGUMENT,
-                    "the chain entry points cover float32, block_size 8 and 1 to 4 inner iterations "
+                    "the chain entry points cover float32, block_size 8 and 1 to 8 inner iterations "
                     "(dtype id %d, block_size %d, inner %d): use gridnet_hip_fused_backward",
                     dtype, block_size, inner);
     if (int rc = check_fused(a, true)) return rc;

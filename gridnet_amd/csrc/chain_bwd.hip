@@ -1,5 +1,5 @@
 // Backward of one step of the network body "update step, then per-sample LayerNorm" inside a
-// CHAIN of such steps: 8^3 blocks, fp32, normalize off, up to 4 inner iterations.
+// CHAIN of such steps: 8^3 blocks, fp32, normalize off, up to 8 inner iterations.
 //
 // The reference's backward scatters what crosses a block boundary into the grid with global
 // atomics (src/gridnet_cuda_kernels.cu:424-435); the tuned kernels of step_fast.hip finish dx in
@@ -44,8 +44,9 @@ namespace gridnet {
 namespace {
 
 constexpr int kShell = 488;  // (8 + 2)^3 - 8^3 window entries around a block
-constexpr int kChainMaxInner = 4;  // the pre-activations of more iterations do not fit: two workgroups
+constexpr int kChainMaxInner = 8;  // the pre-activations of more iterations do not fit: two workgroups
                                     // share the 160 KB of a CU
+constexpr int kChainNarrowInner = 4;  // up to here the table below has its full 24 rows
 constexpr int kChainDepth = 4;  // neighbour rows requested ahead of the arithmetic
 
 // The 488 values a block RECEIVES for one element, by where they come from: the neighbouring
@@ -149,7 +150,7 @@ template <typename T> __device__ __forceinline__ T ld_agent_uniform(const T *p) 
 
 // LDS (floats): [x window x2 | delta window x2 | u_i of the owned cells, inner slabs of 512 |
 // gamma, beta of the window, packed | sums of the four waves | weights of the shell entries
-// [9][512] | per-thread constants [kTab][256]]; at set-up the block's 27 weight planes pass
+// [9][512] | per-thread constants [rows][256]]; at set-up the block's 27 weight planes pass
 // through the front of it.
 using ChainTile = Tile<8, 2>;
 // Table entries.  Small integers are packed (the table is the difference between two workgroups
@@ -157,13 +158,27 @@ using ChainTile = Tile<8, 2>;
 // float indices per word; ShellAt = both shell entries' places in the x window, 16 bits each;
 // Halo = per shell entry the window offset of its centre source (bits 0-11) and the codes of its
 // two strides (bits 12-13, 14-15: 0 -> 1, 1 -> row, 2 -> plane).
-enum { kTabDst = 0, kTabIn = 2, kTabShellAt = 5, kTabHalo = 6, kTabShellGamma = 8, kTabShellBeta = 10,
-       kTabBeta = 12, kTabGamma = 14, kTabAcc = 16 /* 8 gradient sums */, kTab = 24 };
+// WIDE (5 to 8 inner iterations): the history of pre-activations needs the room of eight table
+// rows.  gamma and beta of the owned cells and of the shell entries then come out of the packed
+// gamma/beta window (which holds them anyway: the shell entries are the window's halo) through
+// two rows of offsets, OwnAff and ShellAff (per shell entry 15 bits of offset and a flag: the
+// entry is a row's end entry, whose beta sits 1 float behind its gamma instead of 4), and the
+// pre-activations of the last iteration, which the sweep uses first, stay in registers.
+template <bool WIDE> struct ChainTab {
+    static constexpr int Dst = 0, In = 2, ShellAt = 5, Halo = 6;
+    static constexpr int ShellGamma = 8, ShellBeta = 10, Beta = 12, Gamma = 14;  // narrow only
+    static constexpr int OwnAff = 8, ShellAff = 9;                               // WIDE only
+    static constexpr int Acc = WIDE ? 10 : 16;  // 8 gradient sums
+    static constexpr int Rows = WIDE ? 18 : 24;
+};
 constexpr int kChainAffine = 200 * Fetch<ChainTile>::GB;  // packed gamma/beta: 200 half rows
 __host__ __device__ constexpr int chain_lds_floats(int inner) {
-    const int run = 4 * ChainTile::WIN + inner * 512 + kChainAffine + 16 + 9 * 512 + kTab * 256;
+    const bool wide = inner > kChainNarrowInner;
+    const int run = 4 * ChainTile::WIN + (wide ? inner - 1 : inner) * 512 + kChainAffine + 16 + 9 * 512 +
+                    (wide ? ChainTab<true>::Rows : ChainTab<false>::Rows) * 256;
     return run > 27 * 512 ? run : 27 * 512;
 }
+static_assert(chain_lds_floats(kChainMaxInner) * 4 * 2 <= 160 * 1024, "two workgroups share a CU's LDS");
 __device__ __forceinline__ int stride_of(unsigned code) {
     return code == 0 ? 1 : code == 1 ? ChainTile::RS : ChainTile::PS;
 }
@@ -188,21 +203,25 @@ __device__ __forceinline__ int stride_of(unsigned code) {
 // element ahead, together with the window.  Waits are bounded: a wave that runs out of tries
 // sets the status word and stops waiting for good (results are then invalid, the host falls
 // back to one launch per step), so every workgroup reaches the end whatever happens.
-template <int ACT, bool DEFER, bool ALL = false>
+template <int ACT, bool DEFER, bool ALL = false, bool WIDE = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 void chain_bwd(const ChainBwdArgs a) {
     static_assert(DEFER || !ALL, "inside one launch every step hands its halo values on");
     using TL = ChainTile;
+    using TB = ChainTab<WIDE>;
+    constexpr int kTabDst = TB::Dst, kTabIn = TB::In, kTabShellAt = TB::ShellAt, kTabHalo = TB::Halo,
+                  kTabShellGamma = TB::ShellGamma, kTabShellBeta = TB::ShellBeta, kTabBeta = TB::Beta,
+                  kTabGamma = TB::Gamma, kTabAcc = TB::Acc;
     constexpr int BS = 8, CPT = 2, NC = BS * BS * BS;
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int inner = a.inner;
     float *win = lds;                          // two copies of the x window
     float *dwin = win + 2 * TL::WIN;           // two delta windows, halo zero
     float *hist = dwin + 2 * TL::WIN;          // u_i of this thread's cells at hist + it * 512 + lane * 2
-    float *affine = hist + inner * 512;        // gamma and beta of the window, packed per half row
+    float *affine = hist + (WIDE ? inner - 1 : inner) * 512;  // gamma and beta of the window, packed per half row
     float *red = affine + kChainAffine;   // [2][4][2], per wave: the two LayerNorm sums of an element, elements alternating
     float *hwl = red + 16;                     // [256][18]: the weights that feed the shell entries
-    // ... and what a thread uses once per element: [kTab][256], entry k of thread t at
+    // ... and what a thread uses once per element: [rows][256], entry k of thread t at
     // ctab[k * 256 + t].  The register file has no room for these, and a spilled register is
     // worse than an LDS read: spill traffic queues behind the prefetch in the memory pipeline.
     unsigned *ctab = reinterpret_cast<unsigned *>(hwl + 9 * 512);
@@ -260,7 +279,7 @@ void chain_bwd(const ChainBwdArgs a) {
         // this block's weights pass through LDS once: every thread picks up the mirrored
         // weights of its cells' in-block neighbours and the weights that feed its shell entries
         float hw[2][9], hgam[2], hbet[2];
-        unsigned s_dst[2], s_at[2];
+        unsigned s_dst[2], s_at[2], s_aff[2];
         int h_base[2], h_sb[2], h_sc[2];
         float *wl = lds;  // [27][NC], by block-local cell (i, j, k)
         const int lin = (pl.i * BS + pl.j) * BS + pl.kt * CPT;
@@ -286,6 +305,12 @@ void chain_bwd(const ChainBwdArgs a) {
             const bool ing = have && gi >= 0 && gi < a.M && gj >= 0 && gj < N && gk >= 0 && gk < K;
             s_in[e] = ing;
             s_at[e] = wi * TL::PS + wj * TL::RS + wk;  // the entry in the x window
+            {   // ... and in the packed gamma/beta window: an end entry of its row, or one of its cells
+                const bool is_end = wk == 0 || wk == TL::S - 1;
+                const int half_row = (wi * TL::S + wj) * 2 + (wk >= TL::S / 2 ? 1 : 0);
+                s_aff[e] = (unsigned)(half_row * Fetch<TL>::GB + (is_end ? 2 * Fetch<TL>::HC : (wk - 1) % Fetch<TL>::HC)) |
+                           (is_end ? 1u << 15 : 0u);
+            }
             // the block that owns the cell; the entry's number is its place in that block's record
             const int di = wi == 0 ? -1 : wi == 9 ? 1 : 0, dj = wj == 0 ? -1 : wj == 9 ? 1 : 0,
                       dk = wk == 0 ? -1 : wk == 9 ? 1 : 0;
@@ -323,22 +348,34 @@ void chain_bwd(const ChainBwdArgs a) {
 #pragma unroll
         for (int e = 0; e < 2; ++e)
             tab(kTabHalo + e) = (unsigned)h_base[e] | code_of(h_sb[e]) << 12 | code_of(h_sc[e]) << 14;
-        tab(kTabGamma) = __float_as_uint(gam[0]);
-        tab(kTabGamma + 1) = __float_as_uint(gam[1]);
+        if (!WIDE) {
+            tab(kTabGamma) = __float_as_uint(gam[0]);
+            tab(kTabGamma + 1) = __float_as_uint(gam[1]);
+        } else {
+            // where the packed window keeps gamma of the thread's two cells (beta: 4 floats on)
+            const int half_row = ((pl.i + 1) * TL::S + pl.j + 1) * 2 + (pl.kt >> 1);
+            tab(TB::OwnAff) = (unsigned)(half_row * Fetch<TL>::GB + (pl.kt & 1) * 2);
+        }
         if (DEFER) {
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
 #pragma unroll
                 for (int slot = 0; slot < 9; ++slot) hwl[tid * 18 + e * 9 + slot] = hw[e][slot];
                 tab(kTabDst + e) = s_dst[e];
-                tab(kTabShellGamma + e) = __float_as_uint(hgam[e]);
-                tab(kTabShellBeta + e) = __float_as_uint(hbet[e]);
+                if (!WIDE) {
+                    tab(kTabShellGamma + e) = __float_as_uint(hgam[e]);
+                    tab(kTabShellBeta + e) = __float_as_uint(hbet[e]);
+                }
             }
             tab(kTabShellAt) = s_at[0] | s_at[1] << 16;
-            float bet[CPT];
-            load_cells<CPT>(a.beta + pl.gc, bet);
-            tab(kTabBeta) = __float_as_uint(bet[0]);
-            tab(kTabBeta + 1) = __float_as_uint(bet[1]);
+            if (!WIDE) {
+                float bet[CPT];
+                load_cells<CPT>(a.beta + pl.gc, bet);
+                tab(kTabBeta) = __float_as_uint(bet[0]);
+                tab(kTabBeta + 1) = __float_as_uint(bet[1]);
+            } else {
+                tab(TB::ShellAff) = s_aff[0] | s_aff[1] << 16;
+            }
         }
     }
 
@@ -365,7 +402,7 @@ void chain_bwd(const ChainBwdArgs a) {
     const unsigned ugc = 4u * pl.gc;  // byte offset of the owned cells within a sample
 
     typename Fetch<TL>::Buf pre;
-    if (ln_in) {  // gamma and beta of the window, once per workgroup
+    if (ln_in || WIDE) {  // gamma and beta of the window, once per workgroup
         typename Fetch<TL>::Buf bet;
         fx.fetch(a.gamma, pre);
         fx.fetch(a.beta, bet);
@@ -485,8 +522,18 @@ void chain_bwd(const ChainBwdArgs a) {
 #pragma unroll
                 for (int slot = 0; slot < 9; ++slot)
                     acc = fmaf(hwv[e * 9 + slot], src[(slot / 3 - 1) * sb + (slot % 3 - 1) * sc], acc);
-                t1 = fmaf(__uint_as_float(tab(kTabShellGamma + e)), acc, t1);
-                t2 = fmaf(acc, nh_done[e] - __uint_as_float(tab(kTabShellBeta + e)), t2);
+                float gam_at, bet_at;  // gamma and beta at the cell that receives the value
+                if (WIDE) {
+                    const unsigned code = (tab(TB::ShellAff) >> (16 * e)) & 0xffffu;
+                    const float *at = affine + (code & 0x7fffu);
+                    gam_at = at[0];
+                    bet_at = (code >> 15) ? at[1] : at[Fetch<TL>::HC];
+                } else {
+                    gam_at = __uint_as_float(tab(kTabShellGamma + e));
+                    bet_at = __uint_as_float(tab(kTabShellBeta + e));
+                }
+                t1 = fmaf(gam_at, acc, t1);
+                t2 = fmaf(acc, nh_done[e] - bet_at, t2);
                 if (s_in[e]) {
                     // opaque here, so that the offset is widened inside this block, where the
                     // store can still take it as a 32-bit lane offset beside the scalar base
@@ -521,7 +568,7 @@ void chain_bwd(const ChainBwdArgs a) {
         done_s = -1;
     };
 
-    if (ln_in) lds_barrier();  // the packed gamma and beta
+    if (ln_in || WIDE) lds_barrier();  // the packed gamma and beta
     // ALL: `ready_word` is the ready word of the item at hand's counterpart in the step after
     // (item n - B), requested while the element before was worked on.  `duty` is the next item this
     // workgroup is in charge of (blk, blk + nblk, ...), `duty_count` what its counter read an
@@ -662,13 +709,17 @@ void chain_bwd(const ChainBwdArgs a) {
         shell_of_done(shc, n);
 
         // ---- forward recompute; u_i of the owned cells is remembered ----
-        float xcur[CPT];
+        float xcur[CPT], u_last[CPT] = {0.f, 0.f};  // WIDE: the last iteration's pre-activations
 #pragma unroll
         for (int c = 0; c < CPT; ++c) xcur[c] = win[pl.own + c];
         for (int it = 0; it < inner; ++it) {
             float u[CPT];
             stencil<TL, CPT, kChainDepth>(win + (it & 1) * TL::WIN, pl.row00, w, bv, u);
-            store_cells<CPT>(hist + it * 512 + tid * CPT, u);
+            if (!WIDE || it + 1 < inner) store_cells<CPT>(hist + it * 512 + tid * CPT, u);
+            if (WIDE) {
+#pragma unroll
+                for (int c = 0; c < CPT; ++c) u_last[c] = u[c];
+            }
 #pragma unroll
             for (int c = 0; c < CPT; ++c) {
                 xcur[c] = fmaf(rv[c], Act<ACT, float>::f(u[c]), xcur[c]);
@@ -694,12 +745,21 @@ void chain_bwd(const ChainBwdArgs a) {
             tot[0] += fk == 0 ? ends : 0.f;
             tot[1] += fk == 1 ? ends : 0.f;
             const float yr[CPT] = {yr2.x, yr2.y};
+            float gm[CPT];
+            if (WIDE) {
+                const float2 g2 = *reinterpret_cast<const float2 *>(affine + tab(TB::OwnAff));
+                gm[0] = g2.x;
+                gm[1] = g2.y;
+            } else {
+                gm[0] = __uint_as_float(tab(kTabGamma));
+                gm[1] = __uint_as_float(tab(kTabGamma + 1));
+            }
 #pragma unroll
             for (int c = 0; c < CPT; ++c) {
                 const float yh = (yr[c] - ny0) * ny1;
                 acc_ref(4 + c) = fmaf(tot[c], yh, acc_ref(4 + c));
                 acc_ref(6 + c) += tot[c];
-                g[c] = ny1 * (__uint_as_float(tab(kTabGamma + c)) * tot[c] - ny2 - yh * ny3);
+                g[c] = ny1 * (gm[c] * tot[c] - ny2 - yh * ny3);
                 dsum[c] = 0.f;
             }
         }
@@ -709,7 +769,12 @@ void chain_bwd(const ChainBwdArgs a) {
         float nh[2] = {0.f, 0.f}, dre[CPT] = {0.f, 0.f};
         for (int it = inner - 1; it >= 0; --it) {
             float u[CPT];
-            load_cells<CPT>(hist + it * 512 + tid * CPT, u);
+            if (WIDE && it == inner - 1) {
+#pragma unroll
+                for (int c = 0; c < CPT; ++c) u[c] = u_last[c];
+            } else {
+                load_cells<CPT>(hist + it * 512 + tid * CPT, u);
+            }
 #pragma unroll
             for (int c = 0; c < CPT; ++c) {
                 float f, d;
@@ -764,8 +829,19 @@ void chain_bwd(const ChainBwdArgs a) {
             // cells' share of the two LayerNorm sums
 #pragma unroll
             for (int c = 0; c < CPT; ++c) dwin[TL::WIN + pl.own + c] = dsum[c];
-            const float bet0 = __uint_as_float(tab(kTabBeta)), bet1 = __uint_as_float(tab(kTabBeta + 1));
-            t1_done = fmaf(__uint_as_float(tab(kTabGamma)), g[0], __uint_as_float(tab(kTabGamma + 1)) * g[1]);
+            float bet0, bet1, gam0, gam1;
+            if (WIDE) {
+                const float *at = affine + tab(TB::OwnAff);
+                const float2 g2 = *reinterpret_cast<const float2 *>(at);
+                const float2 b2 = *reinterpret_cast<const float2 *>(at + Fetch<TL>::HC);
+                gam0 = g2.x; gam1 = g2.y; bet0 = b2.x; bet1 = b2.y;
+            } else {
+                bet0 = __uint_as_float(tab(kTabBeta));
+                bet1 = __uint_as_float(tab(kTabBeta + 1));
+                gam0 = __uint_as_float(tab(kTabGamma));
+                gam1 = __uint_as_float(tab(kTabGamma + 1));
+            }
+            t1_done = fmaf(gam0, g[0], gam1 * g[1]);
             t2_done = fmaf(g[0], xcur[0] - bet0, g[1] * (xcur[1] - bet1));
             nh_done[0] = nh[0];
             nh_done[1] = nh[1];
@@ -820,8 +896,8 @@ void chain_bwd(const ChainBwdArgs a) {
     commit_grads<1, CPT>((a.dbeta + slab_off), one, a.param_mode, own_cell, always);
 }
 
-template <int ACT, bool DEFER> int launch_chain(const StepArgs &a, hipStream_t st) {
-    auto kern = chain_bwd<ACT, DEFER>;
+template <int ACT, bool DEFER, bool WIDE> int launch_chain(const StepArgs &a, hipStream_t st) {
+    auto kern = chain_bwd<ACT, DEFER, false, WIDE>;
     const size_t lds = (size_t)chain_lds_floats(a.inner) * sizeof(float);
     static bool big_lds_enabled = false;           // per instantiation
     static int per_cu_cache[kChainMaxInner + 1];   // per instantiation, by inner iterations
@@ -945,8 +1021,8 @@ ChainAllLayout chain_all_layout(const ChainAll &c) {
     return l;
 }
 
-template <int ACT> int launch_chain_all(const ChainAll &c, hipStream_t st) {
-    auto kern = chain_bwd<ACT, true, true>;
+template <int ACT, bool WIDE> int launch_chain_all(const ChainAll &c, hipStream_t st) {
+    auto kern = chain_bwd<ACT, true, true, WIDE>;
     const size_t lds = (size_t)chain_lds_floats(c.inner) * sizeof(float);
     static bool big_lds_enabled = false;
     if (lds > 64 * 1024 && !big_lds_enabled) {
@@ -997,7 +1073,9 @@ template <int ACT> int launch_chain_all(const ChainAll &c, hipStream_t st) {
 }
 
 template <int ACT> int dispatch_defer(const StepArgs &a, hipStream_t st) {
-    return a.ln.halo_out ? launch_chain<ACT, true>(a, st) : launch_chain<ACT, false>(a, st);
+    if (a.inner > kChainNarrowInner)
+        return a.ln.halo_out ? launch_chain<ACT, true, true>(a, st) : launch_chain<ACT, false, true>(a, st);
+    return a.ln.halo_out ? launch_chain<ACT, true, false>(a, st) : launch_chain<ACT, false, false>(a, st);
 }
 
 }  // namespace
@@ -1022,10 +1100,11 @@ bool chain_all_supports(int B, int M, int N, int K, int inner, int outer) {
     static int per_cu_cache[kChainMaxInner + 1];
     int &per_cu = per_cu_cache[inner];
     if (per_cu == 0) {
-        auto kern = chain_bwd<GRIDNET_ACT_LEAKY_RELU, true, true>;
+        const void *kern = inner > kChainNarrowInner ? (const void *)chain_bwd<GRIDNET_ACT_LEAKY_RELU, true, true, true>
+                                                     : (const void *)chain_bwd<GRIDNET_ACT_LEAKY_RELU, true, true, false>;
         const size_t lds = (size_t)chain_lds_floats(inner) * sizeof(float);
         if (lds > 64 * 1024 &&
-            hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize,
+            hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize,
                                 (int)((size_t)chain_lds_floats(kChainMaxInner) * sizeof(float))) != hipSuccess)
             return false;
         int n = 0;
@@ -1039,12 +1118,16 @@ bool chain_all_supports(int B, int M, int N, int K, int inner, int outer) {
 
 size_t chain_all_workspace(const ChainAll &c) { return chain_all_layout(c).total; }
 
+template <int ACT> int dispatch_all(const ChainAll &c, hipStream_t st) {
+    return c.inner > kChainNarrowInner ? launch_chain_all<ACT, true>(c, st) : launch_chain_all<ACT, false>(c, st);
+}
+
 int chain_backward_all(const ChainAll &c, hipStream_t st) {
     switch (c.activation) {
-        case GRIDNET_ACT_RELU: return launch_chain_all<GRIDNET_ACT_RELU>(c, st);
-        case GRIDNET_ACT_LEAKY_RELU: return launch_chain_all<GRIDNET_ACT_LEAKY_RELU>(c, st);
-        case GRIDNET_ACT_SILU: return launch_chain_all<GRIDNET_ACT_SILU>(c, st);
-        case GRIDNET_ACT_TANH: return launch_chain_all<GRIDNET_ACT_TANH>(c, st);
+        case GRIDNET_ACT_RELU: return dispatch_all<GRIDNET_ACT_RELU>(c, st);
+        case GRIDNET_ACT_LEAKY_RELU: return dispatch_all<GRIDNET_ACT_LEAKY_RELU>(c, st);
+        case GRIDNET_ACT_SILU: return dispatch_all<GRIDNET_ACT_SILU>(c, st);
+        case GRIDNET_ACT_TANH: return dispatch_all<GRIDNET_ACT_TANH>(c, st);
     }
     return fail(GRIDNET_ERR_ACTIVATION, "unknown activation function: id %d", c.activation);
 }

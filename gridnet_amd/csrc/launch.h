@@ -108,7 +108,7 @@ int step_fast_backward_parts(int block_size);  // (sum g, sum g*xhat) pairs
 int step_cross_launch(const StepArgs &a, int nchunk, int chunk_len, hipStream_t st);
 
 // chain_bwd.hip: backward of one step of a chain with the cross-block part deferred to the step
-// before (a.ln.halo_in / halo_out); fp32, 8^3 blocks, 1..4 inner iterations, normalize off
+// before (a.ln.halo_in / halo_out); fp32, 8^3 blocks, 1..8 inner iterations, normalize off
 bool chain_supports(const StepArgs &a);
 size_t chain_halo_floats(const StepArgs &a);
 int chain_backward(const StepArgs &a, hipStream_t st);

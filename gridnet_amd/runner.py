@@ -10,7 +10,7 @@ step kernels: a step reads the raw output of the step before it and normalises i
 loading, so the LayerNorm costs no pass over the activations of its own (one, for the final
 output).  Same results within rounding; fp32, ``normalize=False``, ``inner >= 1`` only.
 
-With ``fused=True`` and a problem it covers (float32, 8^3 blocks, up to 4 inner iterations) the
+With ``fused=True`` and a problem it covers (float32, 8^3 blocks, up to 8 inner iterations) the
 backward of a chain goes through ``gridnet_hip_chain_backward``
 (``chain=True``, the default): the backward hands what crosses a block boundary from step to
 step instead of finishing every dx (one kernel per step instead of two).  Same results to

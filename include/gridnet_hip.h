@@ -277,7 +277,7 @@ int gridnet_hip_fused_backward_residual(int dtype, const void *weight, const voi
  * (element, block), in halo_out [B, nblk, 488]; the call for the step BEFORE takes that buffer as
  * its halo_in and adds the values while it loads its incoming gradient.  One kernel per step
  * instead of two, and no scratch tensor written and read back.
- * float32, normalize = false, block_size 8, 1 <= inner <= 4; gridnet_hip_chain_supported() tells,
+ * float32, normalize = false, block_size 8, 1 <= inner <= 8; gridnet_hip_chain_supported() tells,
  * other problems use gridnet_hip_fused_backward.  Results agree with it to rounding.
  */
 int gridnet_hip_chain_supported(int dtype, int inner, int block_size, int normalize);
@@ -316,7 +316,7 @@ int gridnet_hip_chain_backward(int dtype, const void *weight, const void *bias, 
  *   dy      [B,M,N,K]        gradient with respect to LayerNorm(y_raw[outer-1])
  *   dweight, dbias, dscale, dgamma, dbeta   accumulated, or written with GRIDNET_OVERWRITE_PARAMS
  *   dx      [B,M,N,K]        gradient with respect to x0, fully written
- * float32, normalize = false, block_size 8, 1 <= inner <= 4, outer >= 2, B >= 6, and a grid whose
+ * float32, normalize = false, block_size 8, 1 <= inner <= 8, outer >= 2, B >= 6, and a grid whose
  * blocks all fit the GPU at once (M/8 * N/8 * K/8 workgroups resident: 512 on an MI355X, a 64^3
  * grid); gridnet_hip_chain_all_supported() tells.  Results agree with the chain of
  * gridnet_hip_chain_backward calls to rounding and are the same bits on every run.

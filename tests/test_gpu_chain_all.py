@@ -49,13 +49,15 @@ def workload(grid, batch, inner, outer, activation):
 # smooth activations: the comparison of gradients is entry by entry (tests/helpers.py on kinks)
 @pytest.mark.parametrize("grid,batch,inner,outer,activation", [
     (16, 6, 2, 2, "silu"), (16, 7, 4, 3, "tanh"), (32, 6, 2, 3, "silu"), (32, 9, 1, 4, "tanh"),
-    (16, 33, 3, 2, "silu")])
+    (16, 33, 3, 2, "silu"), (16, 6, 8, 3, "tanh"), (32, 7, 5, 2, "silu")])
 def test_one_launch_chain_matches_oracle(grid, batch, inner, outer, activation):
     from gridnet_amd.configs import make_inputs
 
     wl = workload(grid, batch, inner, outer, activation)
     print(f"one-launch chain grid={grid} batch={batch} inner={inner} outer={outer} act={activation}", flush=True)
     t = randomise_affine(make_inputs(wl, seed=3))
+    if inner >= 5:  # keep that many residual updates contractive (fp32 rounding otherwise grows)
+        t["weight"], t["scale"] = t["weight"] * 0.5, t["scale"] * 0.5
     got = run_chain(wl, t, True)
     again = run_chain(wl, t, True)
     for name, g, e in zip(NAMES, got, again):
@@ -151,7 +153,8 @@ def test_unsupported_problems_are_refused():
     assert sup(n.F32, 32, 64, 64, 64, 4, 12, 8, 0) == 1
     assert sup(n.F32, 32, 128, 128, 128, 4, 12, 8, 0) == 0   # 4096 blocks are not resident at once
     assert sup(n.F32, 5, 64, 64, 64, 4, 12, 8, 0) == 0       # batch below the minimum
-    assert sup(n.F32, 32, 64, 64, 64, 5, 12, 8, 0) == 0      # inner iterations
+    assert sup(n.F32, 32, 64, 64, 64, 8, 12, 8, 0) == 1      # the reference's ImageNet default shape
+    assert sup(n.F32, 32, 64, 64, 64, 9, 12, 8, 0) == 0      # inner iterations
     assert sup(n.F32, 32, 64, 64, 64, 4, 1, 8, 0) == 0       # a chain has at least two steps
     assert sup(n.F64, 32, 64, 64, 64, 4, 12, 8, 0) == 0
     assert sup(n.F32, 32, 64, 64, 64, 4, 12, 4, 0) == 0

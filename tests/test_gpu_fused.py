@@ -233,6 +233,10 @@ def test_fused_full_size_agrees_with_op_by_op_chain():
                                            # plain stores on the last step, read-add-write on the others
     ((64, 64, 64), 2, 4, 2, "leaky_relu"), # the same plan under the workloads' own activation (forward only)
     ((8, 8, 8), 4, 2, 3, "relu"),          # a single block: nothing crosses a boundary
+    ((16, 16, 16), 3, 5, 2, "tanh"),       # 5 to 8 inner iterations: the kernels' wide variant (the
+    ((16, 24, 8), 2, 8, 3, "silu"),        # history of pre-activations takes the room of table rows)
+    ((32, 32, 32), 2, 7, 2, "silu"),
+    ((16, 16, 16), 2, 8, 1, "tanh"),
     ((16, 16, 16), 2, 4, 1, "silu"),       # one outer step: the call that finishes dx itself
 ])
 def test_chain_backward_matches_fused_backward(shape, batch, inner, outer, activation):
@@ -246,6 +250,8 @@ def test_chain_backward_matches_fused_backward(shape, batch, inner, outer, activ
     print(f"chain vs fused backward shape={shape} B={batch} inner={inner} outer={outer} act={activation}",
           flush=True)
     w, b, r = make_params(shape, seed=61)
+    if inner >= 7:  # keep that many residual updates contractive (fp32 rounding otherwise grows)
+        w, r = w * 0.5, r * 0.5
     g = torch.Generator().manual_seed(62)
     gamma = 1 + 0.2 * torch.randn(shape, generator=g)
     beta = 0.2 * torch.randn(shape, generator=g)
@@ -272,15 +278,19 @@ def test_chain_backward_matches_fused_backward(shape, batch, inner, outer, activ
                                        inner_iterations=inner, outer_iterations=outer, block_size=8,
                                        activation=activation, normalize=False)
         if activation not in KINKED:
+            # parameter gradients are fp32 sums of batch x inner x outer terms: as elsewhere in this
+            # file their atol is scaled from the bar's own cases (two terms) by sqrt(terms / 2)
+            summed = 1e-5 * max(1.0, (batch * inner * outer / 2) ** 0.5)
             for name_, a, e in zip(NAMES, results[1], exp):
-                assert_close(a, e, what=name_)
+                assert_close(a, e, what=name_, atol=summed if name_ in ("dweight", "dbias", "dscale", "dgamma", "dbeta") else 1e-5)
 
 
 def test_chain_entry_point_rejects_what_it_does_not_cover():
     from gridnet_amd import native as n
 
     assert n.lib.gridnet_hip_chain_supported(n.F32, 4, 8, 0) == 1
-    assert n.lib.gridnet_hip_chain_supported(n.F32, 5, 8, 0) == 0   # the LDS holds 4 iterations
+    assert n.lib.gridnet_hip_chain_supported(n.F32, 8, 8, 0) == 1   # the reference's ImageNet default
+    assert n.lib.gridnet_hip_chain_supported(n.F32, 9, 8, 0) == 0   # the LDS holds the history of 8
     assert n.lib.gridnet_hip_chain_supported(n.F32, 4, 4, 0) == 0   # 8^3 blocks only
     assert n.lib.gridnet_hip_chain_supported(n.F64, 4, 8, 0) == 0
     assert n.lib.gridnet_hip_chain_supported(n.F32, 4, 8, 1) == 0
@@ -293,7 +303,7 @@ def test_chain_entry_point_rejects_what_it_does_not_cover():
                                           p, None, 1, 8, 8, 8, 2, 8, 2, 0, p, 1 << 20, n.current_stream(x))
     assert rc != 0 and "halo_out" in n.last_error()
     rc = n.lib.gridnet_hip_chain_backward(n.F32, p, p, p, p, p, p, None, p, p, p, p, None, None, p, p, p, p, p,
-                                          p, None, 1, 8, 8, 8, 5, 8, 2, 0, p, 1 << 20, n.current_stream(x))
+                                          p, None, 1, 8, 8, 8, 9, 8, 2, 0, p, 1 << 20, n.current_stream(x))
     assert rc != 0 and "inner" in n.last_error()
     rc = n.lib.gridnet_hip_chain_backward(n.F32, p, p, p, p, p, p, None, p, p, p, p, None, None, p, p, p, p, p,
                                           p, None, 1, 8, 8, 8, 2, 8, 2, 0, p, 0, n.current_stream(x))
