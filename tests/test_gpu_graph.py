@@ -12,17 +12,21 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-@pytest.mark.parametrize("fused", [False, True])
-def test_graph_replays_match_eager(fused):
+# one_launch: the chain backward as ONE cooperative launch of resident workgroups that signal each
+# other through counters in the workspace (cleared by a kernel in front of every launch)
+@pytest.mark.parametrize("fused,one_launch", [(False, False), (True, False), (True, True)])
+def test_graph_replays_match_eager(fused, one_launch):
     from gridnet_amd.configs import WORKLOADS, make_inputs
     from gridnet_amd.runner import BodyRunner
     import dataclasses
 
-    wl = dataclasses.replace(WORKLOADS["C3"], batch=4, outer=3)
-    print(f"graph replay: {wl.name} with batch 4 outer 3 fused={fused}", flush=True)
+    wl = dataclasses.replace(WORKLOADS["C3"], batch=8 if one_launch else 4, outer=3)
+    print(f"graph replay: {wl.name} with batch {wl.batch} outer 3 fused={fused} one_launch={one_launch}", flush=True)
     t = {k: v.to(DEV) for k, v in make_inputs(wl, seed=0).items()}
     run = BodyRunner(t["weight"], t["bias"], t["scale"], t["gamma"], t["beta"], wl.batch, wl.inner,
-                     wl.outer, wl.block_size, wl.activation, wl.normalize, backward=True, fused=fused)
+                     wl.outer, wl.block_size, wl.activation, wl.normalize, backward=True, fused=fused,
+                     chain_all=one_launch)
+    assert run.chain_all == one_launch
     x0, gy = t["x0"].clone(), t["grad_out"].clone()
 
     def one_step():
@@ -60,3 +64,4 @@ def test_graph_replays_match_eager(fused):
                                   outs, want):
             # every sum has a fixed order (also where the batch is split over workgroups): same bits
             assert torch.equal(got, exp), f"replay {rep}: {name} differs from the eager result"
+        assert run.chain_all_status() == 0
