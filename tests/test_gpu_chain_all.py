@@ -72,6 +72,36 @@ def test_one_launch_chain_matches_oracle(grid, batch, inner, outer, activation):
         assert_close(g, e, what=name, atol=1e-5 * (terms / 64) ** 0.5 if summed else 1e-5)
 
 
+@pytest.mark.parametrize("shape,batch,inner,outer", [((16, 24, 8), 6, 2, 3), ((8, 16, 40), 7, 3, 2), ((8, 8, 8), 6, 1, 2)])
+def test_one_launch_chain_on_grids_that_are_not_cubes(shape, batch, inner, outer):
+    """M, N and K differ (and a single block along an axis has no neighbour there): the records'
+    addressing and the row-wise completion of dx at the end must not depend on a cubic grid."""
+    from gridnet_amd.runner import BodyRunner
+    from helpers import make_acts, make_params
+    from oracle.network import network_forward_backward
+
+    print(f"one-launch chain shape={shape} B={batch} inner={inner} outer={outer}", flush=True)
+    w, b, r = make_params(shape, seed=71)
+    g = torch.Generator().manual_seed(72)
+    gamma = 1 + 0.2 * torch.randn(shape, generator=g)
+    beta = 0.2 * torch.randn(shape, generator=g)
+    x0, gy = make_acts(batch, shape, seed=73), make_acts(batch, shape, seed=74)
+    results = []
+    for one_launch in (False, True):
+        run = BodyRunner(*(v.to(DEV) for v in (w, b, r, gamma, beta)), batch, inner, outer, 8, "silu", False,
+                         backward=True, fused=True, chain_all=one_launch)
+        assert run.chain_all == one_launch
+        y = run.forward(x0.to(DEV)).clone()
+        results.append((y, *[v.clone() for v in run.backward(gy.to(DEV))]))
+        assert run.chain_all_status() == 0
+    exp = network_forward_backward([v.double() for v in (w, b, r, gamma, beta)], x0.double(), gy.double(),
+                                   inner_iterations=inner, outer_iterations=outer, block_size=8,
+                                   activation="silu", normalize=False)
+    for name, a, e, o in zip(NAMES, results[1], results[0], exp):
+        assert_close(a, e.double(), what=name + " vs launch per step")
+        assert_close(a, o, what=name)
+
+
 def test_one_launch_chain_accumulates_into_the_gradient_buffers():
     """Without GRIDNET_OVERWRITE_PARAMS the parameter gradients are added to what the buffers hold."""
     from gridnet_amd import native as n
