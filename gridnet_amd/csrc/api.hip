@@ -477,8 +477,7 @@ static int fused_backward(int dtype, const void *weight, const void *bias, const
     a.ln.g_rows = g_out ? (const float *)g_out : (const float *)dy;
     if (int rc = step_backward_fast(a, st)) return rc;
     if (!x_stats) return GRIDNET_OK;
-    const int nblk = (M / block_size) * (N / block_size) * (K / block_size);
-    return layernorm_finalize_sums(a.ln.x_part, nblk * step_fast_backward_parts(block_size),
+    return layernorm_finalize_sums(a.ln.x_part, step_fast_backward_pairs(a),
                                    (long)M * N * K, (float *)x_sums, B, st);
 }
 
@@ -573,8 +572,7 @@ int gridnet_hip_chain_backward(int dtype, const void *weight, const void *bias, 
     a.ln.g_rows = (const float *)dy;
     if (int rc = chain_backward(a, st)) return rc;
     if (!x_stats) return GRIDNET_OK;
-    const int nblk = (M / block_size) * (N / block_size) * (K / block_size);
-    return layernorm_finalize_sums(a.ln.x_part, nblk * step_fast_backward_parts(block_size),
+    return layernorm_finalize_sums(a.ln.x_part, step_fast_backward_pairs(a),
                                    (long)M * N * K, (float *)x_sums, B, st);
 }
 

@@ -101,7 +101,15 @@ int step_backward_fast(const StepArgs &a, hipStream_t st);
 // partial statistics per (block, batch element) that the kernels above write when asked to
 int step_fast_forward_parts(int block_size);   // (mean, M2) pairs, each over forward_part_count cells
 int step_fast_forward_part_count(int block_size);
-int step_fast_backward_parts(int block_size);  // (sum g, sum g*xhat) pairs
+int step_fast_backward_parts(int block_size);  // (sum g, sum g*xhat) pairs, at most
+int step_fast_backward_pairs(const StepArgs &a);  // pairs per sample that the backward of `a` leaves
+
+// cross_rows.hip: the cross-block part of the backward for 4^3 blocks, dealt by whole K-rows
+// (a.workspace holds D, a.dx the block-local part; LayerNorm fold as a.ln says); K of 16, 32, 64
+// or 128, normalize off
+bool cross_rows_supports(const StepArgs &a);
+int cross_rows_pairs(const StepArgs &a);  // LayerNorm sum pairs per sample that it leaves in a.ln.x_part
+int cross_rows_launch(const StepArgs &a, hipStream_t st);
 
 // step_fast.hip: the cross-block kernel alone (8^3 blocks, folded LayerNorm arguments in a.ln, the
 // D tensor in a.workspace), for chain_bwd.hip

@@ -1817,6 +1817,7 @@ int launch_bwd_ln(const StepArgs &a, hipStream_t st) {
     // same blocks, same batch chunks; the parameter gradients are complete, dx is not yet
     constexpr int XSLOT = BS == 8 ? kCrossSlots8 : kCrossSlots4;
     constexpr int XE = BS == 8 ? kCrossElems8 : kCrossElems4;
+    if (BS == 4 && cross_rows_supports(a)) return cross_rows_launch(a, st);
     hipLaunchKernelGGL((step_bwd_cross<BS, XSLOT, XE, LN, RES, NORM>), dim3(padded_grid(p.nblk, p.nchunk)),
                        dim3(6 * BS * BS * XSLOT), 0, st, (const float *)a.weight,
                        (const float *)a.x, (const float *)a.workspace, (float *)a.dx, a.B, a.M, a.N,
@@ -1897,6 +1898,10 @@ int step_fast_forward_part_count(int block_size) {
     return block_size * block_size * block_size / step_fast_forward_parts(block_size);
 }
 int step_fast_backward_parts(int) { return 1; }
+int step_fast_backward_pairs(const StepArgs &a) {
+    if (cross_rows_supports(a)) return cross_rows_pairs(a);
+    return (a.M / a.block_size) * (a.N / a.block_size) * (a.K / a.block_size);
+}
 
 bool step_fast_supports(const StepArgs &a, bool backward) {
     if (a.dtype != GRIDNET_F32) return false;
