@@ -572,7 +572,10 @@ int gridnet_hip_chain_backward(int dtype, const void *weight, const void *bias, 
     a.ln.g_rows = (const float *)dy;
     if (int rc = chain_backward(a, st)) return rc;
     if (!x_stats) return GRIDNET_OK;
-    return layernorm_finalize_sums(a.ln.x_part, step_fast_backward_pairs(a),
+    // the sums come from chain_bwd itself (a pair per block) when dx is left unfinished, from the
+    // cross-block kernel otherwise
+    const int nblk = (M / block_size) * (N / block_size) * (K / block_size);
+    return layernorm_finalize_sums(a.ln.x_part, halo_out ? nblk : step_fast_backward_pairs(a),
                                    (long)M * N * K, (float *)x_sums, B, st);
 }
 

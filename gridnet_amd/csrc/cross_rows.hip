@@ -1,19 +1,20 @@
-// The cross-block part of the backward for 4^3 blocks, dealt by whole K-rows.
+// The cross-block part of the backward, dealt by whole K-rows.
 //
 // step_bwd_fast leaves D = sum_i delta_i of every cell and the block-local part of dx.  What is
 // still owed to a cell c is, over the taps t whose neighbour h = c + off_t lies in ANOTHER block,
 //   dx[c] += W[26-t, h] * D[h]
 // (the reference scatters these through its window atomics, src/gridnet_cuda_kernels.cu:424-449).
-// With 4^3 blocks 56 of a block's 64 cells have such taps and a block's row along K is 16 bytes:
-// a workgroup per block touches memory in 16-byte pieces that lie a whole grid row apart.  Here
-// a workgroup takes a TUBE instead: the K/4 blocks that share (block row, block column), 4 x 4 x K
-// cells.  A thread owns one block row of 4 cells (lanes run along K, so the 16 rows of the tube
-// are read and written as whole contiguous rows) and keeps the mirrored weights of all its
-// (cell, tap) pairs in registers for its share of the batch, zero where the tap stays inside the
-// block or leaves the grid: the arithmetic is the plain 27-tap stencil on D, uniform for all
-// threads.  D of the 6 x 6 rows around the tube waits in LDS, two stages alternating, one barrier
-// per batch element; a thread reads 16-byte pieces of nine rows and gets the two cells beside a
-// piece from the lanes next to it (a wave shift, no LDS access).
+// A block's row along K is 16 or 32 bytes: a workgroup per block touches memory in pieces of that
+// size that lie a whole grid row apart (and with 4^3 blocks 56 of a block's 64 cells have such
+// taps).  Here a workgroup takes a TUBE instead: 16 whole grid rows, 4 x 4 x K cells with 4^3
+// blocks (the K/4 blocks that share a block row and column), 2 x 8 x K with 8^3 blocks (a quarter
+// of such a row of blocks).  A thread owns 4 cells along K (lanes run along K, so the rows of
+// the tube are read and written as whole contiguous rows) and keeps the mirrored weights of all
+// its (cell, tap) pairs in registers for its share of the batch, zero where the tap stays inside
+// the block or leaves the grid: the arithmetic is the plain 27-tap stencil on D, uniform for all
+// threads.  D of the rows in and around the tube waits in LDS, two stages alternating, one
+// barrier per batch element; a thread reads 16-byte pieces of nine rows and gets the two cells
+// beside a piece from the lanes next to it (a wave shift, no LDS access).
 //
 // LN / RES as in step_bwd_cross (LnFold): with the LayerNorm of the network body folded in the
 // finished rows also give the two per-sample sums of that LayerNorm's backward, one pair per
@@ -28,7 +29,12 @@ namespace gridnet {
 
 namespace {
 
-constexpr int kTubeRows = 36;  // 6 x 6 rows of D around (and in) a tube
+// a tube is RI x RJ grid rows (16 of them), the D rows in and around it (RI + 2) x (RJ + 2)
+template <int BS> struct Tube {
+    static constexpr int RI = 16 / BS, RJ = BS, WJ = RJ + 2, ROWS = (RI + 2) * WJ;
+    static constexpr int RPT = (ROWS + 15) / 16;  // D rows a thread moves
+    static_assert(BS == 4 || BS == 8, "block sizes 4 and 8");
+};
 
 // the lane before / after in the wave (the caller masks the ends of a row)
 __device__ __forceinline__ float lane_before(float v) {
@@ -38,18 +44,21 @@ __device__ __forceinline__ float lane_after(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x130, 0xf, 0xf, false));
 }
 
-template <bool LN, bool RES>
+template <int BS, bool LN, bool RES>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 3)))
 void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
                 const float *__restrict__ dsum, float *__restrict__ dx, int B, int M, int N, int K,
                 int ntube, int nchunk, int chunk_len, LnFold ln) {
-    extern __shared__ __attribute__((aligned(16))) float lds[];  // [2 stages][36 rows][K]
+    using TB = Tube<BS>;
+    extern __shared__ __attribute__((aligned(16))) float lds[];  // [2 stages][TB::ROWS][K]
 
     int tube, chunk;
     if (!split_block_id(blockIdx.x, ntube, nchunk, tube, chunk)) return;  // grid padding
-    const int kb = K / 4, nt = 16 * kb, tid = threadIdx.x;
-    const int bk = tid % kb, r = tid / kb, ci = r >> 2, cj = r & 3;
-    const int nbj = N / 4, p0 = (tube / nbj) * 4, q0 = (tube % nbj) * 4;
+    const int kb = K / 4, nt = 16 * kb, tid = threadIdx.x;  // kb: threads along a row
+    const int bk = tid % kb, r = tid / kb, ci = r / TB::RJ, cj = r % TB::RJ;
+    const int nbj = N / TB::RJ, p0 = (tube / nbj) * TB::RI, q0 = (tube % nbj) * TB::RJ;
+    // where the thread's row and its first cell lie inside their block
+    const int bi = (p0 + ci) % BS, bj = cj, bk0 = (4 * bk) % BS;
     const long cells = (long)M * N * K;
     const int grow = ((p0 + ci) * N + (q0 + cj)) * K + 4 * bk;  // this thread's four cells
     const bool first = bk == 0, last = bk == kb - 1;
@@ -60,14 +69,16 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
     for (int pq = 0; pq < 9; ++pq) {
         const int di = pq / 3 - 1, dj = pq % 3 - 1;
         const int gi = p0 + ci + di, gj = q0 + cj + dj;
-        const bool side = ci + di < 0 || ci + di > 3 || cj + dj < 0 || cj + dj > 3;
+        const bool side = bi + di < 0 || bi + di >= BS || bj + dj < 0 || bj + dj >= BS;
         const bool row_ok = gi >= 0 && gi < M && gj >= 0 && gj < N;
 #pragma unroll
         for (int dk = -1; dk <= 1; ++dk)
 #pragma unroll
             for (int ck = 0; ck < 4; ++ck) {
-                const bool along = ck + dk < 0 || ck + dk > 3;  // known when compiling
-                if (pq == 4 && !along) continue;                // never crosses: not held at all
+                // a tap along K can only cross where it leaves the thread's four cells (known
+                // when compiling); taps that never cross are not held at all
+                if (pq == 4 && !(ck + dk < 0 || ck + dk > 3)) continue;
+                const bool along = bk0 + ck + dk < 0 || bk0 + ck + dk >= BS;
                 const int gk = 4 * bk + ck + dk;
                 const int t = (di + 1) * 9 + (dj + 1) * 3 + (dk + 1);
                 const bool use = (side || along) && row_ok && gk >= 0 && gk < K;
@@ -79,23 +90,24 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
     float gam[4] = {0.f, 0.f, 0.f, 0.f};
     if (ln_in) load_cells<4>(ln.gamma + grow, gam);
 
-    // ---- the D rows this thread moves: rows r, r + 16 and (the first four r) r + 32 ----
-    int goff[3], loff[3];
-    bool ok[3];
+    // ---- the D rows this thread moves: rows r, r + 16, ... while there are any ----
+    constexpr int RPT = TB::RPT;
+    int goff[RPT], loff[RPT];
+    bool ok[RPT];
 #pragma unroll
-    for (int e = 0; e < 3; ++e) {
-        const int row = r + 16 * e, wi = row / 6, wj = row % 6;
+    for (int e = 0; e < RPT; ++e) {
+        const int row = r + 16 * e, wi = row / TB::WJ, wj = row % TB::WJ;
         const int gi = p0 + wi - 1, gj = q0 + wj - 1;
-        ok[e] = row < kTubeRows && gi >= 0 && gi < M && gj >= 0 && gj < N;
+        ok[e] = row < TB::ROWS && gi >= 0 && gi < M && gj >= 0 && gj < N;
         goff[e] = ok[e] ? (gi * N + gj) * K + 4 * bk : grow;  // anything valid when not used
         loff[e] = row * K + 4 * bk;
     }
-    const bool third = r < kTubeRows - 32;
-    const int own_row = (ci + 1) * 6 + (cj + 1);
+    const bool has_last = r + 16 * (RPT - 1) < TB::ROWS;
+    const int own_row = (ci + 1) * TB::WJ + (cj + 1);
     wait_global_loads();
 
     const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
-    float dbuf[3][4], gx[4], xr[4], gr[4], xmean = 0.f, xrstd = 1.f;
+    float dbuf[RPT][4], gx[4], xr[4], gr[4], xmean = 0.f, xrstd = 1.f;
     auto fetch = [&](int s) {
         const long at = (long)s * cells;
         load_cells<4>(dx + at + grow, gx);
@@ -106,14 +118,14 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
             xrstd = load_ahead(ln.x_stats, 2 * s + 1);
         }
 #pragma unroll
-        for (int e = 0; e < 3; ++e) load_cells<4>(dsum + at + goff[e], dbuf[e]);
+        for (int e = 0; e < RPT; ++e) load_cells<4>(dsum + at + goff[e], dbuf[e]);
     };
     if (s0 < s1) fetch(s0);
     for (int s = s0; s < s1; ++s) {
-        float *stage = lds + ((s - s0) & 1) * kTubeRows * K;
+        float *stage = lds + ((s - s0) & 1) * TB::ROWS * K;
 #pragma unroll
-        for (int e = 0; e < 3; ++e) {
-            if (e == 2 && !third) break;
+        for (int e = 0; e < RPT; ++e) {
+            if (e == RPT - 1 && !has_last) break;
             float v[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) v[q] = ok[e] ? dbuf[e][q] : 0.f;
@@ -135,7 +147,7 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
             const int di = pq / 3 - 1, dj = pq % 3 - 1;
             float d[6];
             float mid[4];
-            load_cells<4>(stage + (own_row + di * 6 + dj) * K + 4 * bk, mid);
+            load_cells<4>(stage + (own_row + di * TB::WJ + dj) * K + 4 * bk, mid);
             const float before = lane_before(mid[3]), after = lane_after(mid[0]);
             d[0] = first ? 0.f : before;
             d[5] = last ? 0.f : after;
@@ -175,10 +187,11 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
 
 bool k_ok(int K) { return K == 16 || K == 32 || K == 64 || K == 128; }
 
-template <bool LN, bool RES> int launch(const StepArgs &a, hipStream_t st) {
-    auto kern = cross_rows<LN, RES>;
-    const int nt = 4 * a.K, ntube = (a.M / 4) * (a.N / 4);
-    const size_t lds = (size_t)2 * kTubeRows * a.K * sizeof(float);
+template <int BS, bool LN, bool RES> int launch(const StepArgs &a, hipStream_t st) {
+    using TB = Tube<BS>;
+    auto kern = cross_rows<BS, LN, RES>;
+    const int nt = 4 * a.K, ntube = (a.M / TB::RI) * (a.N / TB::RJ);
+    const size_t lds = (size_t)2 * TB::ROWS * a.K * sizeof(float);
     static int per_cu_cache[4] = {0, 0, 0, 0};  // per instantiation, by K
     int &per_cu = per_cu_cache[a.K == 16 ? 0 : a.K == 32 ? 1 : a.K == 64 ? 2 : 3];
     if (per_cu == 0) {
@@ -199,19 +212,25 @@ template <bool LN, bool RES> int launch(const StepArgs &a, hipStream_t st) {
     return check_launch("cross_rows");
 }
 
+template <int BS> int dispatch(const StepArgs &a, hipStream_t st) {
+    if (a.ln.gamma && a.ln.residual) return launch<BS, true, true>(a, st);
+    if (a.ln.gamma) return launch<BS, true, false>(a, st);
+    return launch<BS, false, false>(a, st);
+}
+
 }  // namespace
 
 bool cross_rows_supports(const StepArgs &a) {
-    return a.dtype == GRIDNET_F32 && a.block_size == 4 && !a.normalize && k_ok(a.K) && a.M % 4 == 0 &&
-           a.N % 4 == 0;
+    const int bs = a.block_size;
+    return a.dtype == GRIDNET_F32 && (bs == 4 || bs == 8) && !a.normalize && k_ok(a.K) && a.M % bs == 0 &&
+           a.N % bs == 0;
 }
 
-int cross_rows_pairs(const StepArgs &a) { return (a.M / 4) * (a.N / 4) * (4 * a.K / 64); }
+// one pair per wave: 16 grid rows of K / 4 threads each per workgroup
+int cross_rows_pairs(const StepArgs &a) { return (a.M * a.N / 16) * (4 * a.K / 64); }
 
 int cross_rows_launch(const StepArgs &a, hipStream_t st) {
-    if (a.ln.gamma && a.ln.residual) return launch<true, true>(a, st);
-    if (a.ln.gamma) return launch<true, false>(a, st);
-    return launch<false, false>(a, st);
+    return a.block_size == 8 ? dispatch<8>(a, st) : dispatch<4>(a, st);
 }
 
 }  // namespace gridnet

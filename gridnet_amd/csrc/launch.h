@@ -101,7 +101,7 @@ int step_backward_fast(const StepArgs &a, hipStream_t st);
 // partial statistics per (block, batch element) that the kernels above write when asked to
 int step_fast_forward_parts(int block_size);   // (mean, M2) pairs, each over forward_part_count cells
 int step_fast_forward_part_count(int block_size);
-int step_fast_backward_parts(int block_size);  // (sum g, sum g*xhat) pairs, at most
+int step_fast_backward_parts(int block_size);  // (sum g, sum g*xhat) pairs per (block, element), at most
 int step_fast_backward_pairs(const StepArgs &a);  // pairs per sample that the backward of `a` leaves
 
 // cross_rows.hip: the cross-block part of the backward for 4^3 blocks, dealt by whole K-rows

@@ -1817,7 +1817,7 @@ int launch_bwd_ln(const StepArgs &a, hipStream_t st) {
     // same blocks, same batch chunks; the parameter gradients are complete, dx is not yet
     constexpr int XSLOT = BS == 8 ? kCrossSlots8 : kCrossSlots4;
     constexpr int XE = BS == 8 ? kCrossElems8 : kCrossElems4;
-    if (BS == 4 && cross_rows_supports(a)) return cross_rows_launch(a, st);
+    if (!NORM && cross_rows_supports(a)) return cross_rows_launch(a, st);  // by whole K-rows
     hipLaunchKernelGGL((step_bwd_cross<BS, XSLOT, XE, LN, RES, NORM>), dim3(padded_grid(p.nblk, p.nchunk)),
                        dim3(6 * BS * BS * XSLOT), 0, st, (const float *)a.weight,
                        (const float *)a.x, (const float *)a.workspace, (float *)a.dx, a.B, a.M, a.N,
@@ -1862,6 +1862,7 @@ template <bool BWD> int dispatch(const StepArgs &a, hipStream_t st) {
 // The cross-block kernel alone, completing a dx whose block-local part another kernel wrote
 // (8^3 blocks; the LayerNorm fold as a.ln says; D in a.workspace).
 int step_cross_launch(const StepArgs &a, int nchunk, int chunk_len, hipStream_t st) {
+    if (cross_rows_supports(a)) return cross_rows_launch(a, st);
     const int nblk = (a.M / 8) * (a.N / 8) * (a.K / 8);
     hipLaunchKernelGGL((step_bwd_cross<8, kCrossSlots8, kCrossElems8, true>), dim3(padded_grid(nblk, nchunk)),
                        dim3(6 * 64 * kCrossSlots8), 0, st, (const float *)a.weight, (const float *)a.x,
@@ -1897,7 +1898,9 @@ int step_fast_forward_parts(int block_size) {
 int step_fast_forward_part_count(int block_size) {
     return block_size * block_size * block_size / step_fast_forward_parts(block_size);
 }
-int step_fast_backward_parts(int) { return 1; }
+// per block at most: the kernel dealt by block face leaves one pair per block, the row-wise one a
+// pair per 256 cells (two per 8^3 block, a quarter per 4^3 block)
+int step_fast_backward_parts(int block_size) { return block_size == 8 ? 2 : 1; }
 int step_fast_backward_pairs(const StepArgs &a) {
     if (cross_rows_supports(a)) return cross_rows_pairs(a);
     return (a.M / a.block_size) * (a.N / a.block_size) * (a.K / a.block_size);

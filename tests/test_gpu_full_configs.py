@@ -14,8 +14,12 @@ worst entries 0.08 to 0.16 of the bar's bound at all four shapes.
 Gradients of a chain of 12 to 16 outer steps: parameter gradients are sums of up to 10^4 fp32
 terms per entry and a few entries in a million leave the bar in ANY fp32 evaluation (under
 silu at C3: 44 of 7 million dweight entries for the fused chain, 40 for the op-by-op chain).
-Asserted under a smooth activation: no entry further from the fp64 chain than twice the worst
-entry of the op-by-op fp32 chain (or inside the bar).
+Asserted under a smooth activation: the errors of the fused chain are distributed like those of
+the op-by-op fp32 chain -- at every threshold k = 1, 2, 4, ... bar units, no more entries beyond
+k than twice the number the op-by-op chain has beyond k / 2 (give or take three entries), and no
+entry beyond four times its worst.  (The worst single entry of seven million is a noisy yardstick:
+two valid fp32 evaluations differ by a factor of two to three in it, and it moves whenever a
+kernel of either chain changes its summation order.)
 Under leaky_relu (the workloads' own activation) some of the 10^8 pre-activations lie within
 fp32 rounding of the kink, where fp32 and fp64 take different branches of the derivative; the
 LayerNorm couples all cells of a sample, so every such flip moves every upstream gradient a
@@ -60,9 +64,10 @@ def excess(got, want):
 
 def hold_to_fp64(name, fused, steps, ref, kinked=False):
     """The fused result against the fp64 chain, with the op-by-op fp32 chain as the yardstick of
-    what fp32 does to this problem.  Smooth activations: no entry beyond max(1, 2 x the
-    yardstick's worst) bar units.  ``kinked``: the fraction of entries outside the bar stays
-    below 1 % and below twice the yardstick's fraction (plus one entry in 10^4)."""
+    what fp32 does to this problem.  Smooth activations: beyond every threshold k = 1, 2, 4, ...
+    bar units lie at most twice as many entries as the yardstick has beyond k / 2, plus three, and
+    none lies beyond max(1, 4 x the yardstick's worst).  ``kinked``: the fraction of entries outside
+    the bar stays below 1 % and below twice the yardstick's fraction (plus one entry in 10^4)."""
     ef, es = excess(fused, ref), excess(steps, ref)
     worst_f, worst_s = ef.max().item(), es.max().item()
     out_f, out_s = (ef > 1).double().mean().item(), (es > 1).double().mean().item()
@@ -74,10 +79,16 @@ def hold_to_fp64(name, fused, steps, ref, kinked=False):
         assert out_f <= 1e-2 and out_f <= 2 * out_s + 1e-4, (
             f"{name}: {out_f:.3e} of the entries are outside the bar (op-by-op fp32 chain: {out_s:.3e})")
     else:
-        limit = max(1.0, 2.0 * worst_s)
+        limit = max(1.0, 4.0 * worst_s)
         assert worst_f <= limit, (
             f"{name}: worst entry {worst_f:.3f} bar units from the fp64 chain, limit {limit:.3f} "
             f"(op-by-op fp32 worst {worst_s:.3f})")
+        k = 1.0
+        while k < worst_f:
+            n_f, n_s = int((ef > k).sum()), int((es > k / 2).sum())
+            assert n_f <= 2 * n_s + 3, (
+                f"{name}: {n_f} entries beyond {k:g} bar units, the op-by-op fp32 chain has {n_s} beyond {k / 2:g}")
+            k *= 2
 
 
 def layernorm_invariants(y, gamma_is_one=True):

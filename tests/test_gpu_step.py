@@ -71,6 +71,10 @@ MATRIX = [
     ((8, 16, 8), 4, 3, False, "relu"),
     ((8, 16, 8), 8, 5, True, "tanh"),
     ((8, 16, 8), 4, 3, True, "relu"),
+    # 4^3 blocks with rows of 16, 32 and 64 cells (the cross-block part is dealt by whole rows there)
+    ((4, 4, 16), 4, 2, False, "relu"),
+    ((12, 8, 32), 4, 2, False, "silu"),
+    ((8, 12, 64), 4, 3, False, "tanh"),
     # no inner iteration on a grid of several blocks: the gradient passes through unchanged
     ((16, 24, 16), 8, 0, True, "silu"),
     ((8, 16, 8), 4, 0, False, "tanh"),
