@@ -19,6 +19,10 @@
 // LN / RES as in step_bwd_cross (LnFold): with the LayerNorm of the network body folded in the
 // finished rows also give the two per-sample sums of that LayerNorm's backward, one pair per
 // wave; the residual loop's G' is subtracted from the rows first.
+// NORM (per-window normalisation, see step_bwd_fast): `dsum` holds D1, and a cell that lies in the
+// halo of a neighbouring block a additionally receives R_a - x Q_a, with (Q, R) the two numbers
+// per (element, block) that step_bwd_fast left in `qr`.  All threads of a tube have the same 3 x 3
+// columns of blocks around them: their (Q, R) travel through LDS with the D rows.
 
 #include "common.h"
 #include "fast_tiles.h"
@@ -44,13 +48,15 @@ __device__ __forceinline__ float lane_after(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x130, 0xf, 0xf, false));
 }
 
-template <int BS, bool LN, bool RES>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 3)))
+template <int BS, bool LN, bool RES, bool NORM = false>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3, 3)))
 void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
                 const float *__restrict__ dsum, float *__restrict__ dx, int B, int M, int N, int K,
-                int ntube, int nchunk, int chunk_len, LnFold ln) {
+                int ntube, int nchunk, int chunk_len, LnFold ln, const float *__restrict__ qr) {
     using TB = Tube<BS>;
-    extern __shared__ __attribute__((aligned(16))) float lds[];  // [2 stages][TB::ROWS][K]
+    static_assert(!(NORM && (LN || RES)), "the folded LayerNorm comes without normalisation");
+    // [2 stages][TB::ROWS][K]; NORM: then [2 stages][3 x 3 columns of blocks][K / BS + 2] (Q, R) pairs
+    extern __shared__ __attribute__((aligned(16))) float lds[];
 
     int tube, chunk;
     if (!split_block_id(blockIdx.x, ntube, nchunk, tube, chunk)) return;  // grid padding
@@ -104,14 +110,45 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
     }
     const bool has_last = r + 16 * (RPT - 1) < TB::ROWS;
     const int own_row = (ci + 1) * TB::WJ + (cj + 1);
+
+    // NORM: (Q, R) of the blocks in the 3 x 3 columns around the tube's own, a row of K / BS blocks
+    // each with a zero pair at either end; thread n < 9 K / BS moves one pair per element
+    const int nbk = K / BS, qrow = nbk + 2;
+    float2 *qrs = reinterpret_cast<float2 *>(lds + 2 * TB::ROWS * K);  // [2][9][qrow]
+    long qr_from = -1;
+    int qr_to = 0;
+    // which columns hold blocks that have this thread's row in their halo (beside its own), and
+    // where its own block sits in a row of pairs
+    const int ei = bi == 0 ? -1 : bi == BS - 1 ? 1 : 0, ej = bj == 0 ? -1 : bj == BS - 1 ? 1 : 0;
+    const int kcol = 4 * bk / BS + 1;
+    if (NORM) {
+        const int nblk_j = N / BS, col_i = p0 / BS, col_j = q0 / BS;
+        if (tid < 9 * nbk) {
+            const int a = tid / (3 * nbk), b = (tid / nbk) % 3, kk = tid % nbk;
+            const int gi = col_i + a - 1, gj = col_j + b - 1;
+            qr_to = (a * 3 + b) * qrow + kk + 1;
+            if (gi >= 0 && gi < M / BS && gj >= 0 && gj < nblk_j) qr_from = ((long)gi * nblk_j + gj) * nbk + kk;
+        }
+        if (tid < 36) {  // the zero pairs at the ends of the rows, both stages, once
+            const int st = tid / 18, row = (tid % 18) / 2, end = tid & 1;
+            qrs[(st * 9 + row) * qrow + (end ? qrow - 1 : 0)] = make_float2(0.f, 0.f);
+        }
+    }
     wait_global_loads();
 
     const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
     float dbuf[RPT][4], gx[4], xr[4], gr[4], xmean = 0.f, xrstd = 1.f;
+    float2 qbuf = make_float2(0.f, 0.f);
+    const long nblk = (long)(M / BS) * (N / BS) * nbk;
     auto fetch = [&](int s) {
         const long at = (long)s * cells;
         load_cells<4>(dx + at + grow, gx);
         if (RES) load_cells<4>(ln.g_rows + at + grow, gr);
+        if (NORM) {
+            load_cells<4>(x + at + grow, xr);
+            // (every thread loads, a valid address always; the commit selects)
+            qbuf = *reinterpret_cast<const float2 *>(qr + (s * nblk + (qr_from >= 0 ? qr_from : 0)) * 2);
+        }
         if (ln_in) {
             load_cells<4>(x + at + grow, xr);
             xmean = load_ahead(ln.x_stats, 2 * s);
@@ -131,12 +168,15 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
             for (int q = 0; q < 4; ++q) v[q] = ok[e] ? dbuf[e][q] : 0.f;
             store_cells<4>(stage + loff[e], v);
         }
+        const float2 *qst = qrs + ((s - s0) & 1) * 9 * qrow;
+        if (NORM && tid < 9 * nbk)
+            qrs[((s - s0) & 1) * 9 * qrow + qr_to] = qr_from >= 0 ? qbuf : make_float2(0.f, 0.f);
         float g[4], xc[4], grc[4];
         const float mean = xmean, rstd = xrstd;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             g[c] = gx[c];
-            xc[c] = ln_in ? xr[c] : 0.f;
+            xc[c] = (ln_in || NORM) ? xr[c] : 0.f;
             grc[c] = RES ? gr[c] : 0.f;
         }
         lds_barrier();  // the stage is complete; the readers of the other one are done
@@ -165,6 +205,33 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
 #pragma unroll
             for (int c = 0; c < 4; ++c) g[c] -= grc[c];
         }
+        if (NORM) {
+            // blocks that have the cell in their halo, by their offset along K: the columns
+            // (0, 0), (ei, 0), (0, ej), (ei, ej) as far as the row lies on that side of its block;
+            // at offset 0 the block itself is left out, offsets -1 / +1 concern the cell at that
+            // end of the block only
+            float sq[3] = {0.f, 0.f, 0.f}, sr[3] = {0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ia = 0; ia < 2; ++ia)
+#pragma unroll
+                for (int ib = 0; ib < 2; ++ib) {
+                    const bool use = (ia == 0 || ei != 0) && (ib == 0 || ej != 0);
+                    const float2 *row = qst + ((1 + ia * ei) * 3 + (1 + ib * ej)) * qrow + kcol;
+#pragma unroll
+                    for (int dk = 0; dk < 3; ++dk) {
+                        if (dk == 1 && ia == 0 && ib == 0) continue;
+                        const float2 v = row[dk - 1];
+                        sq[dk] += use ? v.x : 0.f;
+                        sr[dk] += use ? v.y : 0.f;
+                    }
+                }
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                g[c] += fmaf(-xc[c], sq[1], sr[1]);
+                if (c == 0 && bk0 == 0) g[c] += fmaf(-xc[c], sq[0], sr[0]);
+                if (c == 3 && bk0 + 3 == BS - 1) g[c] += fmaf(-xc[c], sq[2], sr[2]);
+            }
+        }
         store_cells<4>(dx + (long)s * cells + grow, g);
         if (ln_in) {
             float t1 = 0.f, t2 = 0.f;
@@ -187,11 +254,13 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
 
 bool k_ok(int K) { return K == 16 || K == 32 || K == 64 || K == 128; }
 
-template <int BS, bool LN, bool RES> int launch(const StepArgs &a, hipStream_t st) {
+template <int BS, bool LN, bool RES, bool NORM = false> int launch(const StepArgs &a, hipStream_t st) {
     using TB = Tube<BS>;
-    auto kern = cross_rows<BS, LN, RES>;
+    auto kern = cross_rows<BS, LN, RES, NORM>;
     const int nt = 4 * a.K, ntube = (a.M / TB::RI) * (a.N / TB::RJ);
-    const size_t lds = (size_t)2 * TB::ROWS * a.K * sizeof(float);
+    const size_t lds = ((size_t)2 * TB::ROWS * a.K + (NORM ? 2 * 9 * (a.K / BS + 2) * 2 : 0)) * sizeof(float);
+    // NORM: (Q, R) per (element, block) behind the D tensor in the workspace
+    const float *qr = NORM ? (const float *)a.workspace + (size_t)a.B * a.M * a.N * a.K : nullptr;
     static int per_cu_cache[4] = {0, 0, 0, 0};  // per instantiation, by K
     int &per_cu = per_cu_cache[a.K == 16 ? 0 : a.K == 32 ? 1 : a.K == 64 ? 2 : 3];
     if (per_cu == 0) {
@@ -208,11 +277,12 @@ template <int BS, bool LN, bool RES> int launch(const StepArgs &a, hipStream_t s
     nchunk = (a.B + chunk_len - 1) / chunk_len;
     hipLaunchKernelGGL(kern, dim3(padded_grid(ntube, nchunk)), dim3(nt), lds, st, (const float *)a.weight,
                        (const float *)a.x, (const float *)a.workspace, (float *)a.dx, a.B, a.M, a.N, a.K,
-                       ntube, nchunk, chunk_len, a.ln);
+                       ntube, nchunk, chunk_len, a.ln, qr);
     return check_launch("cross_rows");
 }
 
 template <int BS> int dispatch(const StepArgs &a, hipStream_t st) {
+    if (a.normalize) return launch<BS, false, false, true>(a, st);
     if (a.ln.gamma && a.ln.residual) return launch<BS, true, true>(a, st);
     if (a.ln.gamma) return launch<BS, true, false>(a, st);
     return launch<BS, false, false>(a, st);
@@ -222,8 +292,8 @@ template <int BS> int dispatch(const StepArgs &a, hipStream_t st) {
 
 bool cross_rows_supports(const StepArgs &a) {
     const int bs = a.block_size;
-    return a.dtype == GRIDNET_F32 && (bs == 4 || bs == 8) && !a.normalize && k_ok(a.K) && a.M % bs == 0 &&
-           a.N % bs == 0;
+    return a.dtype == GRIDNET_F32 && (bs == 4 || bs == 8) && !(a.normalize && a.ln.gamma) && k_ok(a.K) &&
+           a.M % bs == 0 && a.N % bs == 0;
 }
 
 // one pair per wave: 16 grid rows of K / 4 threads each per workgroup

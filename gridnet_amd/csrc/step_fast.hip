@@ -1817,7 +1817,7 @@ int launch_bwd_ln(const StepArgs &a, hipStream_t st) {
     // same blocks, same batch chunks; the parameter gradients are complete, dx is not yet
     constexpr int XSLOT = BS == 8 ? kCrossSlots8 : kCrossSlots4;
     constexpr int XE = BS == 8 ? kCrossElems8 : kCrossElems4;
-    if (!NORM && cross_rows_supports(a)) return cross_rows_launch(a, st);  // by whole K-rows
+    if (cross_rows_supports(a)) return cross_rows_launch(a, st);  // by whole K-rows
     hipLaunchKernelGGL((step_bwd_cross<BS, XSLOT, XE, LN, RES, NORM>), dim3(padded_grid(p.nblk, p.nchunk)),
                        dim3(6 * BS * BS * XSLOT), 0, st, (const float *)a.weight,
                        (const float *)a.x, (const float *)a.workspace, (float *)a.dx, a.B, a.M, a.N,

@@ -75,6 +75,9 @@ MATRIX = [
     ((4, 4, 16), 4, 2, False, "relu"),
     ((12, 8, 32), 4, 2, False, "silu"),
     ((8, 12, 64), 4, 3, False, "tanh"),
+    ((8, 12, 64), 4, 3, True, "tanh"),
+    ((16, 8, 32), 8, 2, True, "silu"),
+    ((8, 4, 16), 4, 2, True, "relu"),
     # no inner iteration on a grid of several blocks: the gradient passes through unchanged
     ((16, 24, 16), 8, 0, True, "silu"),
     ((8, 16, 8), 4, 0, False, "tanh"),
