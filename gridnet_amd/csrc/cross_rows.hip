@@ -23,6 +23,8 @@
 // halo of a neighbouring block a additionally receives R_a - x Q_a, with (Q, R) the two numbers
 // per (element, block) that step_bwd_fast left in `qr`.  All threads of a tube have the same 3 x 3
 // columns of blocks around them: their (Q, R) travel through LDS with the D rows.
+// SETS = 2: the gated variant of the update (weight [27, 2, M, N, K]): two D tensors, one behind
+// the other in `dsum`, each with its own set of mirrored weights; the cell receives the sum.
 
 #include "common.h"
 #include "fast_tiles.h"
@@ -48,14 +50,15 @@ __device__ __forceinline__ float lane_after(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x130, 0xf, 0xf, false));
 }
 
-template <int BS, bool LN, bool RES, bool NORM = false>
-__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(3, 3)))
+template <int BS, bool LN, bool RES, bool NORM = false, int SETS = 1>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(SETS == 1 ? 3 : 2, SETS == 1 ? 3 : 2)))
 void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
                 const float *__restrict__ dsum, float *__restrict__ dx, int B, int M, int N, int K,
                 int ntube, int nchunk, int chunk_len, LnFold ln, const float *__restrict__ qr) {
     using TB = Tube<BS>;
     static_assert(!(NORM && (LN || RES)), "the folded LayerNorm comes without normalisation");
-    // [2 stages][TB::ROWS][K]; NORM: then [2 stages][3 x 3 columns of blocks][K / BS + 2] (Q, R) pairs
+    static_assert(SETS == 1 || !(LN || RES || NORM), "the gated update has no variants");
+    // [2 stages][SETS][TB::ROWS][K]; NORM: then [2 stages][3 x 3 columns of blocks][K / BS + 2] (Q, R) pairs
     extern __shared__ __attribute__((aligned(16))) float lds[];
 
     int tube, chunk;
@@ -70,7 +73,7 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
     const bool first = bk == 0, last = bk == kb - 1;
 
     // ---- mirrored weights of the pairs (cell, tap) that cross a block boundary ----
-    float vx[9][3][4];
+    float vx[SETS][9][3][4];
 #pragma unroll
     for (int pq = 0; pq < 9; ++pq) {
         const int di = pq / 3 - 1, dj = pq % 3 - 1;
@@ -89,7 +92,9 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
                 const int t = (di + 1) * 9 + (dj + 1) * 3 + (dk + 1);
                 const bool use = (side || along) && row_ok && gk >= 0 && gk < K;
                 const long h = ((long)gi * N + gj) * K + gk;
-                vx[pq][dk + 1][ck] = use ? weight[(26 - t) * cells + h] : 0.f;
+#pragma unroll
+                for (int k = 0; k < SETS; ++k)
+                    vx[k][pq][dk + 1][ck] = use ? weight[((26 - t) * SETS + k) * cells + h] : 0.f;
             }
     }
     const bool ln_in = LN && ln.x_stats != nullptr;
@@ -114,7 +119,7 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
     // NORM: (Q, R) of the blocks in the 3 x 3 columns around the tube's own, a row of K / BS blocks
     // each with a zero pair at either end; thread n < 9 K / BS moves one pair per element
     const int nbk = K / BS, qrow = nbk + 2;
-    float2 *qrs = reinterpret_cast<float2 *>(lds + 2 * TB::ROWS * K);  // [2][9][qrow]
+    float2 *qrs = reinterpret_cast<float2 *>(lds + 2 * SETS * TB::ROWS * K);  // [2][9][qrow]
     long qr_from = -1;
     int qr_to = 0;
     // which columns hold blocks that have this thread's row in their halo (beside its own), and
@@ -137,7 +142,7 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
     wait_global_loads();
 
     const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
-    float dbuf[RPT][4], gx[4], xr[4], gr[4], xmean = 0.f, xrstd = 1.f;
+    float dbuf[SETS][RPT][4], gx[4], xr[4], gr[4], xmean = 0.f, xrstd = 1.f;
     float2 qbuf = make_float2(0.f, 0.f);
     const long nblk = (long)(M / BS) * (N / BS) * nbk;
     auto fetch = [&](int s) {
@@ -155,19 +160,23 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
             xrstd = load_ahead(ln.x_stats, 2 * s + 1);
         }
 #pragma unroll
-        for (int e = 0; e < RPT; ++e) load_cells<4>(dsum + at + goff[e], dbuf[e]);
+        for (int k = 0; k < SETS; ++k)
+#pragma unroll
+            for (int e = 0; e < RPT; ++e) load_cells<4>(dsum + (long)k * B * cells + at + goff[e], dbuf[k][e]);
     };
     if (s0 < s1) fetch(s0);
     for (int s = s0; s < s1; ++s) {
-        float *stage = lds + ((s - s0) & 1) * TB::ROWS * K;
+        float *stage = lds + ((s - s0) & 1) * SETS * TB::ROWS * K;
 #pragma unroll
-        for (int e = 0; e < RPT; ++e) {
-            if (e == RPT - 1 && !has_last) break;
-            float v[4];
+        for (int k = 0; k < SETS; ++k)
 #pragma unroll
-            for (int q = 0; q < 4; ++q) v[q] = ok[e] ? dbuf[e][q] : 0.f;
-            store_cells<4>(stage + loff[e], v);
-        }
+            for (int e = 0; e < RPT; ++e) {
+                if (e == RPT - 1 && !has_last) break;
+                float v[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) v[q] = ok[e] ? dbuf[k][e][q] : 0.f;
+                store_cells<4>(stage + k * TB::ROWS * K + loff[e], v);
+            }
         const float2 *qst = qrs + ((s - s0) & 1) * 9 * qrow;
         if (NORM && tid < 9 * nbk)
             qrs[((s - s0) & 1) * 9 * qrow + qr_to] = qr_from >= 0 ? qbuf : make_float2(0.f, 0.f);
@@ -183,11 +192,13 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
         fetch(min(s + 1, s1 - 1));
         // fixed order per cell: rows (di, dj) in tap order, along K inside a row
 #pragma unroll
+        for (int k = 0; k < SETS; ++k)
+#pragma unroll
         for (int pq = 0; pq < 9; ++pq) {
             const int di = pq / 3 - 1, dj = pq % 3 - 1;
             float d[6];
             float mid[4];
-            load_cells<4>(stage + (own_row + di * TB::WJ + dj) * K + 4 * bk, mid);
+            load_cells<4>(stage + (k * TB::ROWS + own_row + di * TB::WJ + dj) * K + 4 * bk, mid);
             const float before = lane_before(mid[3]), after = lane_after(mid[0]);
             d[0] = first ? 0.f : before;
             d[5] = last ? 0.f : after;
@@ -198,7 +209,7 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
 #pragma unroll
                 for (int ck = 0; ck < 4; ++ck) {
                     if (pq == 4 && !(ck + dk < 0 || ck + dk > 3)) continue;
-                    g[ck] = fmaf(vx[pq][dk + 1][ck], d[ck + 1 + dk], g[ck]);
+                    g[ck] = fmaf(vx[k][pq][dk + 1][ck], d[ck + 1 + dk], g[ck]);
                 }
         }
         if (RES) {
@@ -254,13 +265,22 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
 
 bool k_ok(int K) { return K == 16 || K == 32 || K == 64 || K == 128; }
 
-template <int BS, bool LN, bool RES, bool NORM = false> int launch(const StepArgs &a, hipStream_t st) {
+template <int BS, bool LN, bool RES, bool NORM = false, int SETS = 1>
+int launch(const StepArgs &a, const float *dsum, hipStream_t st) {
     using TB = Tube<BS>;
-    auto kern = cross_rows<BS, LN, RES, NORM>;
+    auto kern = cross_rows<BS, LN, RES, NORM, SETS>;
     const int nt = 4 * a.K, ntube = (a.M / TB::RI) * (a.N / TB::RJ);
-    const size_t lds = ((size_t)2 * TB::ROWS * a.K + (NORM ? 2 * 9 * (a.K / BS + 2) * 2 : 0)) * sizeof(float);
+    const size_t lds = ((size_t)2 * SETS * TB::ROWS * a.K + (NORM ? 2 * 9 * (a.K / BS + 2) * 2 : 0)) * sizeof(float);
+    static bool big_lds_enabled = false;  // per instantiation
+    if (lds > 64 * 1024 && !big_lds_enabled) {
+        if (hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(GRIDNET_ERR_LAUNCH, "cross_rows: cannot enable %zu bytes of LDS", lds);
+        }
+        big_lds_enabled = true;
+    }
     // NORM: (Q, R) per (element, block) behind the D tensor in the workspace
-    const float *qr = NORM ? (const float *)a.workspace + (size_t)a.B * a.M * a.N * a.K : nullptr;
+    const float *qr = NORM ? dsum + (size_t)a.B * a.M * a.N * a.K : nullptr;
     static int per_cu_cache[4] = {0, 0, 0, 0};  // per instantiation, by K
     int &per_cu = per_cu_cache[a.K == 16 ? 0 : a.K == 32 ? 1 : a.K == 64 ? 2 : 3];
     if (per_cu == 0) {
@@ -276,16 +296,17 @@ template <int BS, bool LN, bool RES, bool NORM = false> int launch(const StepArg
     const int chunk_len = (a.B + nchunk - 1) / nchunk;
     nchunk = (a.B + chunk_len - 1) / chunk_len;
     hipLaunchKernelGGL(kern, dim3(padded_grid(ntube, nchunk)), dim3(nt), lds, st, (const float *)a.weight,
-                       (const float *)a.x, (const float *)a.workspace, (float *)a.dx, a.B, a.M, a.N, a.K,
+                       (const float *)a.x, dsum, (float *)a.dx, a.B, a.M, a.N, a.K,
                        ntube, nchunk, chunk_len, a.ln, qr);
     return check_launch("cross_rows");
 }
 
 template <int BS> int dispatch(const StepArgs &a, hipStream_t st) {
-    if (a.normalize) return launch<BS, false, false, true>(a, st);
-    if (a.ln.gamma && a.ln.residual) return launch<BS, true, true>(a, st);
-    if (a.ln.gamma) return launch<BS, true, false>(a, st);
-    return launch<BS, false, false>(a, st);
+    const float *dsum = (const float *)a.workspace;
+    if (a.normalize) return launch<BS, false, false, true>(a, dsum, st);
+    if (a.ln.gamma && a.ln.residual) return launch<BS, true, true>(a, dsum, st);
+    if (a.ln.gamma) return launch<BS, true, false>(a, dsum, st);
+    return launch<BS, false, false>(a, dsum, st);
 }
 
 }  // namespace
@@ -301,6 +322,16 @@ int cross_rows_pairs(const StepArgs &a) { return (a.M * a.N / 16) * (4 * a.K / 6
 
 int cross_rows_launch(const StepArgs &a, hipStream_t st) {
     return a.block_size == 8 ? dispatch<8>(a, st) : dispatch<4>(a, st);
+}
+
+// the gated update: weight [27, 2, M, N, K], D0 and D1 of every cell behind one another in `dsum`
+bool cross_rows_gated_supports(const StepArgs &a) {
+    const int bs = a.block_size;
+    return a.dtype == GRIDNET_F32 && (bs == 4 || bs == 8) && k_ok(a.K) && a.M % bs == 0 && a.N % bs == 0;
+}
+int cross_rows_gated_launch(const StepArgs &a, const float *dsum, hipStream_t st) {
+    return a.block_size == 8 ? launch<8, false, false, false, 2>(a, dsum, st)
+                             : launch<4, false, false, false, 2>(a, dsum, st);
 }
 
 }  // namespace gridnet

@@ -110,6 +110,8 @@ int step_fast_backward_pairs(const StepArgs &a);  // pairs per sample that the b
 bool cross_rows_supports(const StepArgs &a);
 int cross_rows_pairs(const StepArgs &a);  // LayerNorm sum pairs per sample that it leaves in a.ln.x_part
 int cross_rows_launch(const StepArgs &a, hipStream_t st);
+bool cross_rows_gated_supports(const StepArgs &a);  // the gated update: two weight sets, D0 and D1 in `dsum`
+int cross_rows_gated_launch(const StepArgs &a, const float *dsum, hipStream_t st);
 
 // step_fast.hip: the cross-block kernel alone (8^3 blocks, folded LayerNorm arguments in a.ln, the
 // D tensor in a.workspace), for chain_bwd.hip

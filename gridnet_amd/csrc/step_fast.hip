@@ -1874,6 +1874,7 @@ int step_cross_launch(const StepArgs &a, int nchunk, int chunk_len, hipStream_t 
 // The cross-block kernel for the gated update: D0 and D1 of every cell behind one another in
 // `dsum`, weight [27, 2, M, N, K]; same blocks and batch chunks as the kernel that left them.
 int gated_cross_launch(const StepArgs &a, const float *dsum, int nchunk, int chunk_len, hipStream_t st) {
+    if (cross_rows_gated_supports(a)) return cross_rows_gated_launch(a, dsum, st);
     const int bs = a.block_size;
     const int nblk = (a.M / bs) * (a.N / bs) * (a.K / bs);
     const LnFold none{};
