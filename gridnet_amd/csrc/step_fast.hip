@@ -31,8 +31,9 @@
 //     through D = sum_i delta_i.  The gradient of a weight whose tap reads a halo entry is
 //     x_halo * D: the first kernel adds it once per element.  What the cells of NEIGHBOURING
 //     blocks receive needs the neighbours' D: the first kernel leaves D of every cell in a
-//     scratch tensor and a second kernel (step_bwd_cross), dealt by block face, works it out
-//     from the D window with its real halo and completes dx, in a fixed order.
+//     scratch tensor and a second kernel works it out and completes dx, in a fixed order:
+//     cross_rows (cross_rows.hip), dealt by whole grid rows, for rows of 16, 32, 64 or 128 cells;
+//     step_bwd_cross, dealt by block face from the D window with its real halo, for the rest.
 // Forward with 8^3 blocks: the same mapping over a window stored in two parts, so that every LDS
 // access of the inner loop is aligned and free of bank conflicts (step_fwd_split).
 // Parameter gradients leave the kernel once per workgroup: reduced across slots through LDS and,

@@ -71,3 +71,39 @@ def network_forward_backward(params, x0, grad_out, **kw):
     y = network_forward(*leaves, xin, **kw)
     grads = torch.autograd.grad(y, leaves + [xin], grad_out)
     return (y.detach(), *grads)
+
+
+def network_forward_backward_manual(params, x0, grad_out, inner_iterations, outer_iterations,
+                                    block_size, activation="leaky_relu", normalize=False, eps=1e-5,
+                                    ln_eps=1e-5):
+    """The plain loop (``h = norm(net(h))``) forward and backward WITHOUT autograd: the step's
+    hand-derived backward and the LayerNorm backward of ``oracle.manual``, step by step in
+    reverse.  Same return value as ``network_forward_backward``; it keeps one tensor per outer
+    step instead of autograd's graph, which is what lets it run at the benchmark's full sizes."""
+    from .manual import gridnet_step_backward_manual, layer_norm_backward_manual
+
+    weight, bias, scale, gamma, beta = params
+    inputs, raws = [], []
+    h = x0
+    with torch.no_grad():
+        for _ in range(outer_iterations):
+            inputs.append(h)
+            raw = gridnet_step_fast(weight, bias, scale, h, inner_iterations, block_size, eps, normalize,
+                                    activation)
+            raws.append(raw)
+            h = layer_norm_plain(raw, gamma, beta, ln_eps)
+        y = h
+        dw, db, dr = torch.zeros_like(weight), torch.zeros_like(bias), torch.zeros_like(scale)
+        dgamma, dbeta = torch.zeros_like(gamma), torch.zeros_like(beta)
+        g = grad_out
+        for j in reversed(range(outer_iterations)):
+            g, dg, dbt, _, _ = layer_norm_backward_manual(g, raws[j], gamma, ln_eps)
+            dgamma += dg
+            dbeta += dbt
+            sw, sb, sr, g = gridnet_step_backward_manual(weight, bias, scale, inputs[j], g, inner_iterations,
+                                                         block_size, eps, normalize, activation)
+            dw += sw
+            db += sb
+            dr += sr
+            raws[j] = inputs[j] = None
+    return y, dw, db, dr, dgamma, dbeta, g

@@ -1,7 +1,8 @@
 """Every benchmark configuration at its FULL size, on the path ``bench.py`` times (the chain
 with the LayerNorm folded into the step kernels, fp32).
 
-The CPU oracle cannot reach these sizes in test time.  The arbiter here is the op-by-op chain of
+The CPU oracle takes minutes for a whole workload at these sizes (the last C3 test below runs it
+for three outer steps).  The arbiter here is the op-by-op chain of
 the same library run in fp64 on the same fp32 inputs: the generic kernels (one thread per cell,
 scatter with atomics) and the separate LayerNorm kernels, which share no device code with the
 tuned fp32 kernels and are themselves held to the oracle on the shapes it does reach
@@ -135,6 +136,38 @@ def test_c3_full_fused_gradients_smooth_activation():
     ref = chain(wl, t, torch.float64, False)
     for name, f, s, r in zip(NAMES, fused, steps, ref):
         hold_to_fp64(name, f, s, r)
+
+
+def test_c3_full_size_arbiter_is_held_to_the_cpu_oracle():
+    """The arbiter of this file at the full C3 shape (64^3 grid, 8^3 blocks, batch 32, inner 4) against
+    the CPU oracle itself: the loop without autograd (oracle.network, pinned against autograd in
+    tests/test_oracle_backward.py), fp64, the workload's own leaky_relu, three outer steps (the
+    oracle takes about ten seconds per step at this size).  The fp64 chain on the GPU must agree
+    with it to 1e-9; the fused fp32 chain is then held to the ORACLE the way the tests above hold it
+    to the fp64 chain."""
+    from gridnet_amd.configs import WORKLOADS, make_inputs
+    from oracle.network import network_forward_backward_manual
+
+    import os
+
+    # GRIDNET_FULL_ORACLE=1: all twelve outer steps (about a minute of CPU time)
+    wl = WORKLOADS["C3"] if os.environ.get("GRIDNET_FULL_ORACLE") else dataclasses.replace(WORKLOADS["C3"], outer=3)
+    t = make_inputs(wl)
+    print(f"full size against the CPU oracle: {wl.name} with outer={wl.outer}", flush=True)
+    want = network_forward_backward_manual(
+        [t[k].double() for k in PARAMS], t["x0"].double(), t["grad_out"].double(), wl.inner, wl.outer,
+        wl.block_size, wl.activation, wl.normalize)
+    ref = chain(wl, t, torch.float64, False)
+    for name, a, e in zip(NAMES, ref, want):
+        e = e.to(DEV)
+        err = ((a - e).abs() / (1 + e.abs())).max().item()
+        print(f"  {name:8s} fp64 chain against the oracle: worst {err:.2e} (relative to 1 + |value|)", flush=True)
+        assert err < 1e-9, name
+    fused = chain(wl, t, torch.float32, True)
+    steps = chain(wl, t, torch.float32, False)
+    hold_to_fp64("y", fused[0], steps[0], want[0].to(DEV))
+    for name, f, s_, e in list(zip(NAMES, fused, steps, want))[1:]:
+        hold_to_fp64(name, f, s_, e.to(DEV), kinked=True)
 
 
 def test_c4_full_fused_forward():

@@ -133,3 +133,24 @@ def test_network_is_step_then_norm():
     # every sample leaves a LayerNorm with mean beta-ish and unit-ish spread
     flat = ((y - beta) / gamma).flatten(1)
     assert flat.mean(1).abs().max() < 1e-5 and (flat.var(1, correction=0) - 1).abs().max() < 1e-3
+
+
+@pytest.mark.parametrize("activation,normalize", [("silu", False), ("leaky_relu", False), ("tanh", True)])
+def test_manual_chain_matches_autograd_chain(activation, normalize):
+    """The loop without autograd (what the full-size GPU checks are held to) against autograd of
+    the same loop."""
+    from oracle.network import network_forward_backward, network_forward_backward_manual
+
+    shape, bs, batch, inner, outer = (8, 16, 8), 4, 3, 2, 3
+    w, b, r = make_params(shape, seed=31, dtype=torch.float64)
+    g = torch.Generator().manual_seed(32)
+    gamma = 1 + 0.2 * torch.randn(shape, generator=g, dtype=torch.float64)
+    beta = 0.2 * torch.randn(shape, generator=g, dtype=torch.float64)
+    x0 = make_acts(batch, shape, seed=33, dtype=torch.float64)
+    gy = make_acts(batch, shape, seed=34, dtype=torch.float64)
+    kw = dict(inner_iterations=inner, outer_iterations=outer, block_size=bs, activation=activation,
+              normalize=normalize)
+    want = network_forward_backward([w, b, r, gamma, beta], x0, gy, **kw)
+    got = network_forward_backward_manual([w, b, r, gamma, beta], x0, gy, **kw)
+    for name, a, e in zip(("y", "dweight", "dbias", "dscale", "dgamma", "dbeta", "dx0"), got, want):
+        assert torch.allclose(a, e, rtol=1e-9, atol=1e-11), name
