@@ -27,7 +27,7 @@ LDS_BYTES_PER_CLOCK_PER_CU = 128
 CUS = 256
 
 
-def gpu_run(wl, steps, warmup, fused, graph_replay=True, chain_all=None):
+def gpu_run(wl, steps, warmup, fused, graph_replay=True, chain_all=None, chain=None):
     import torch
 
     from gridnet_amd.configs import make_inputs
@@ -38,7 +38,7 @@ def gpu_run(wl, steps, warmup, fused, graph_replay=True, chain_all=None):
     t = {k: v.to(dev) for k, v in make_inputs(wl, seed=0).items()}
     run = BodyRunner(t["weight"], t["bias"], t["scale"], t["gamma"], t["beta"], wl.batch, wl.inner,
                      wl.outer, wl.block_size, wl.activation, wl.normalize, backward=wl.backward,
-                     fused=fused, chain_all=chain_all)
+                     fused=fused, chain_all=chain_all, chain=chain)
 
     def one_step():
         run.forward(t["x0"])
@@ -252,6 +252,11 @@ def main():
                     help="the backward of the whole chain in one launch of resident workgroups "
                          "(gridnet_hip_chain_backward_all): where it applies and fills the chip, "
                          "wherever it applies, never")
+    ap.add_argument("--chain", choices=("auto", "on", "off"), default="auto",
+                    help="the backward inside a chain as one kernel per step that hands the cross-block "
+                         "values on (gridnet_hip_chain_backward) instead of two kernels per step: where the "
+                         "library's row-wise cross-block kernel does not apply, wherever supported, never "
+                         "(off also rules out --chain-all)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true",
                     help="skip the HIP graph replay (for runs under a counter-collecting profiler)")
@@ -268,7 +273,8 @@ def main():
         wl = dataclasses.replace(wl, normalize=True, name=wl.name + " normalize")
     fused = args.path == "fused" and not wl.normalize and wl.inner >= 1
     wall, graph_s, kernel_s, one_launch = gpu_run(wl, args.steps, args.warmup, fused, not args.no_graph,
-                                      {"auto": None, "on": True, "off": False}[args.chain_all])
+                                      {"auto": None, "on": True, "off": False}[args.chain_all],
+                                      {"auto": None, "on": True, "off": False}[args.chain])
     bytes_ = wl.algorithmic_bytes()
     if fused:  # a fused entry point does the work of the step AND of the LayerNorm beside it
         bytes_["step_fwd"] += bytes_["ln_fwd"]

@@ -11,10 +11,13 @@ loading, so the LayerNorm costs no pass over the activations of its own (one, fo
 output).  Same results within rounding; fp32, ``normalize=False``, ``inner >= 1`` only.
 
 With ``fused=True`` and a problem it covers (float32, 8^3 blocks, up to 8 inner iterations) the
-backward of a chain goes through ``gridnet_hip_chain_backward``
-(``chain=True``, the default): the backward hands what crosses a block boundary from step to
-step instead of finishing every dx (one kernel per step instead of two).  Same results to
-rounding.
+backward of a chain can go through ``gridnet_hip_chain_backward``: the backward hands what
+crosses a block boundary from step to step instead of finishing every dx (one kernel per step
+instead of two).  Same results to rounding.  ``chain=None`` (the default) takes it where the
+two-kernel backward would have to deal its cross-block part by block face (rows of other than 16,
+32, 64 or 128 cells); where that part goes by whole rows the two kernels are the faster pair
+(64^3 grid, batch 32, 12 steps: 3.12 against 3.19 ms per training step).  ``True``: wherever the
+library supports it; ``False``: never (nor the one launch below).
 
 Where the whole grid fits the GPU at once (every block a resident workgroup: a 64^3 grid on an
 MI355X) and the steps share one parameter set, the chain backward is ONE launch
@@ -42,7 +45,7 @@ class BodyRunner:
     def __init__(self, weight, bias, scale, gamma, beta, batch: int, inner: int, outer: int,
                  block_size: int, activation: str = "leaky_relu", normalize: bool = False,
                  eps: float = 1e-5, ln_eps: float = 1e-5, backward: bool = True,
-                 fused: bool = False, outer_residual: bool = False, chain: bool = True,
+                 fused: bool = False, outer_residual: bool = False, chain=None,
                  chain_all=None):
         self.separate = isinstance(weight, (list, tuple))
         if self.separate:
@@ -119,15 +122,17 @@ class BodyRunner:
                 self.fb_ws_bytes = _n.lib.gridnet_hip_fused_workspace_bytes(
                     batch, self.M, self.N, self.K, inner, block_size, 1)
                 self.fb_ws = _n.workspace(self.fb_ws_bytes, dev)
-        self.chain = bool(chain and fused and backward and not outer_residual and
-                          _n.lib.gridnet_hip_chain_supported(self.dt, inner, block_size, self.normalize))
+        chain_ok = bool(chain is not False and fused and backward and not outer_residual and
+                        _n.lib.gridnet_hip_chain_supported(self.dt, inner, block_size, self.normalize))
+        rows = self.K in (16, 32, 64, 128)  # what the row-wise cross-block kernel takes
+        self.chain = chain_ok and (chain is True or not rows)
         if self.chain:
             # two buffers that the backward calls of neighbouring steps hand their cross-block
             # values over in
             nfl = _n.lib.gridnet_hip_chain_halo_floats(batch, self.M, self.N, self.K, block_size)
             self.halo = [torch.empty(nfl, device=dev, dtype=dtype) for _ in range(2 if outer > 1 else 0)]
         self.chain_all = False
-        if self.chain and not self.separate and chain_all is not False and \
+        if chain_ok and not self.separate and chain_all is not False and \
                 _n.lib.gridnet_hip_chain_all_supported(self.dt, batch, self.M, self.N, self.K, inner, outer,
                                                        block_size, self.normalize):
             nblk = (self.M // 8) * (self.N // 8) * (self.K // 8)

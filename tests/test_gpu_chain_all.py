@@ -26,7 +26,7 @@ def runner(wl, t, chain_all):
     d = {k: v.to(DEV) for k, v in t.items() if k != "readout"}
     run = BodyRunner(d["weight"], d["bias"], d["scale"], d["gamma"], d["beta"], t["x0"].shape[0],
                      wl.inner, wl.outer, wl.block_size, wl.activation, wl.normalize,
-                     backward=True, fused=True, chain_all=chain_all)
+                     backward=True, fused=True, chain=True, chain_all=chain_all)
     assert run.chain_all == bool(chain_all)
     return run, d
 
@@ -89,7 +89,7 @@ def test_one_launch_chain_on_grids_that_are_not_cubes(shape, batch, inner, outer
     results = []
     for one_launch in (False, True):
         run = BodyRunner(*(v.to(DEV) for v in (w, b, r, gamma, beta)), batch, inner, outer, 8, "silu", False,
-                         backward=True, fused=True, chain_all=one_launch)
+                         backward=True, fused=True, chain=True, chain_all=one_launch)
         assert run.chain_all == one_launch
         y = run.forward(x0.to(DEV)).clone()
         results.append((y, *[v.clone() for v in run.backward(gy.to(DEV))]))
