@@ -27,7 +27,7 @@ LDS_BYTES_PER_CLOCK_PER_CU = 128
 CUS = 256
 
 
-def gpu_run(wl, steps, warmup, fused, graph_replay=True, chain_all=None, chain=None):
+def gpu_run(wl, steps, warmup, fused, graph_replay=True, chain_all=None, chain=None, outer_residual=False):
     import torch
 
     from gridnet_amd.configs import make_inputs
@@ -38,7 +38,7 @@ def gpu_run(wl, steps, warmup, fused, graph_replay=True, chain_all=None, chain=N
     t = {k: v.to(dev) for k, v in make_inputs(wl, seed=0).items()}
     run = BodyRunner(t["weight"], t["bias"], t["scale"], t["gamma"], t["beta"], wl.batch, wl.inner,
                      wl.outer, wl.block_size, wl.activation, wl.normalize, backward=wl.backward,
-                     fused=fused, chain_all=chain_all, chain=chain)
+                     fused=fused, chain_all=chain_all, chain=chain, outer_residual=outer_residual)
 
     def one_step():
         run.forward(t["x0"])
@@ -257,6 +257,9 @@ def main():
                          "values on (gridnet_hip_chain_backward) instead of two kernels per step: where the "
                          "library's row-wise cross-block kernel does not apply, wherever supported, never "
                          "(off also rules out --chain-all)")
+    ap.add_argument("--outer-residual", action="store_true",
+                    help="the other shape of the loop, n = norm(h); h = h + (net(n) - n) "
+                         "(the reference's --outer_residual); fused entry points only")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true",
                     help="skip the HIP graph replay (for runs under a counter-collecting profiler)")
@@ -271,10 +274,14 @@ def main():
     wl = WORKLOADS[args.workload]
     if args.normalize:
         wl = dataclasses.replace(wl, normalize=True, name=wl.name + " normalize")
+    if args.outer_residual:
+        if args.path != "fused" or wl.normalize:
+            sys.exit("bench.py: --outer-residual runs through the fused entry points (no --path steps, no --normalize)")
+        wl = dataclasses.replace(wl, name=wl.name + " outer_residual")
     fused = args.path == "fused" and not wl.normalize and wl.inner >= 1
     wall, graph_s, kernel_s, one_launch = gpu_run(wl, args.steps, args.warmup, fused, not args.no_graph,
                                       {"auto": None, "on": True, "off": False}[args.chain_all],
-                                      {"auto": None, "on": True, "off": False}[args.chain])
+                                      {"auto": None, "on": True, "off": False}[args.chain], args.outer_residual)
     bytes_ = wl.algorithmic_bytes()
     if fused:  # a fused entry point does the work of the step AND of the LayerNorm beside it
         bytes_["step_fwd"] += bytes_["ln_fwd"]

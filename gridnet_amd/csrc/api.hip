@@ -474,7 +474,6 @@ static int fused_backward(int dtype, const void *weight, const void *bias, const
     a.ln.residual = residual;
     a.ln.g_prev = (const float *)g_prev;
     a.ln.g_out = (float *)g_out;
-    a.ln.g_rows = g_out ? (const float *)g_out : (const float *)dy;
     if (int rc = step_backward_fast(a, st)) return rc;
     if (!x_stats) return GRIDNET_OK;
     return layernorm_finalize_sums(a.ln.x_part, step_fast_backward_pairs(a),
@@ -569,7 +568,6 @@ int gridnet_hip_chain_backward(int dtype, const void *weight, const void *bias, 
     a.ln.x_part = x_stats ? (float *)((char *)workspace + dsum_bytes) : nullptr;
     a.ln.halo_in = (const float *)halo_in;
     a.ln.halo_out = (float *)halo_out;
-    a.ln.g_rows = (const float *)dy;
     if (int rc = chain_backward(a, st)) return rc;
     if (!x_stats) return GRIDNET_OK;
     // the sums come from chain_bwd itself (a pair per block) when dx is left unfinished, from the

@@ -16,9 +16,9 @@
 // barrier per batch element; a thread reads 16-byte pieces of nine rows and gets the two cells
 // beside a piece from the lanes next to it (a wave shift, no LDS access).
 //
-// LN / RES as in step_bwd_cross (LnFold): with the LayerNorm of the network body folded in the
-// finished rows also give the two per-sample sums of that LayerNorm's backward, one pair per
-// wave; the residual loop's G' is subtracted from the rows first.
+// LN as in step_bwd_cross (LnFold): with the LayerNorm of the network body folded in the finished
+// rows also give the two per-sample sums of that LayerNorm's backward, one pair per wave.  (The
+// residual form of the loop needs nothing here: step_bwd_fast takes G' off the cells' own part.)
 // NORM (per-window normalisation, see step_bwd_fast): `dsum` holds D1, and a cell that lies in the
 // halo of a neighbouring block a additionally receives R_a - x Q_a, with (Q, R) the two numbers
 // per (element, block) that step_bwd_fast left in `qr`.  All threads of a tube have the same 3 x 3
@@ -50,14 +50,14 @@ __device__ __forceinline__ float lane_after(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x130, 0xf, 0xf, false));
 }
 
-template <int BS, bool LN, bool RES, bool NORM = false, int SETS = 1>
+template <int BS, bool LN, bool NORM = false, int SETS = 1>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(SETS == 1 ? 3 : 2, SETS == 1 ? 3 : 2)))
 void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
                 const float *__restrict__ dsum, float *__restrict__ dx, int B, int M, int N, int K,
                 int ntube, int nchunk, int chunk_len, LnFold ln, const float *__restrict__ qr) {
     using TB = Tube<BS>;
-    static_assert(!(NORM && (LN || RES)), "the folded LayerNorm comes without normalisation");
-    static_assert(SETS == 1 || !(LN || RES || NORM), "the gated update has no variants");
+    static_assert(!(NORM && LN), "the folded LayerNorm comes without normalisation");
+    static_assert(SETS == 1 || !(LN || NORM), "the gated update has no variants");
     // [2 stages][SETS][TB::ROWS][K]; NORM: then [2 stages][3 x 3 columns of blocks][K / BS + 2] (Q, R) pairs
     extern __shared__ __attribute__((aligned(16))) float lds[];
 
@@ -142,13 +142,12 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
     wait_global_loads();
 
     const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
-    float dbuf[SETS][RPT][4], gx[4], xr[4], gr[4], xmean = 0.f, xrstd = 1.f;
+    float dbuf[SETS][RPT][4], gx[4], xr[4], xmean = 0.f, xrstd = 1.f;
     float2 qbuf = make_float2(0.f, 0.f);
     const long nblk = (long)(M / BS) * (N / BS) * nbk;
     auto fetch = [&](int s) {
         const long at = (long)s * cells;
         load_cells<4>(dx + at + grow, gx);
-        if (RES) load_cells<4>(ln.g_rows + at + grow, gr);
         if (NORM) {
             load_cells<4>(x + at + grow, xr);
             // (every thread loads, a valid address always; the commit selects)
@@ -180,13 +179,12 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
         const float2 *qst = qrs + ((s - s0) & 1) * 9 * qrow;
         if (NORM && tid < 9 * nbk)
             qrs[((s - s0) & 1) * 9 * qrow + qr_to] = qr_from >= 0 ? qbuf : make_float2(0.f, 0.f);
-        float g[4], xc[4], grc[4];
+        float g[4], xc[4];
         const float mean = xmean, rstd = xrstd;
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             g[c] = gx[c];
             xc[c] = (ln_in || NORM) ? xr[c] : 0.f;
-            grc[c] = RES ? gr[c] : 0.f;
         }
         lds_barrier();  // the stage is complete; the readers of the other one are done
         fetch(min(s + 1, s1 - 1));
@@ -211,10 +209,6 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
                     if (pq == 4 && !(ck + dk < 0 || ck + dk > 3)) continue;
                     g[ck] = fmaf(vx[k][pq][dk + 1][ck], d[ck + 1 + dk], g[ck]);
                 }
-        }
-        if (RES) {
-#pragma unroll
-            for (int c = 0; c < 4; ++c) g[c] -= grc[c];
         }
         if (NORM) {
             // blocks that have the cell in their halo, by their offset along K: the columns
@@ -265,10 +259,10 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
 
 bool k_ok(int K) { return K == 16 || K == 32 || K == 64 || K == 128; }
 
-template <int BS, bool LN, bool RES, bool NORM = false, int SETS = 1>
+template <int BS, bool LN, bool NORM = false, int SETS = 1>
 int launch(const StepArgs &a, const float *dsum, hipStream_t st) {
     using TB = Tube<BS>;
-    auto kern = cross_rows<BS, LN, RES, NORM, SETS>;
+    auto kern = cross_rows<BS, LN, NORM, SETS>;
     const int nt = 4 * a.K, ntube = (a.M / TB::RI) * (a.N / TB::RJ);
     const size_t lds = ((size_t)2 * SETS * TB::ROWS * a.K + (NORM ? 2 * 9 * (a.K / BS + 2) * 2 : 0)) * sizeof(float);
     static bool big_lds_enabled = false;  // per instantiation
@@ -303,10 +297,9 @@ int launch(const StepArgs &a, const float *dsum, hipStream_t st) {
 
 template <int BS> int dispatch(const StepArgs &a, hipStream_t st) {
     const float *dsum = (const float *)a.workspace;
-    if (a.normalize) return launch<BS, false, false, true>(a, dsum, st);
-    if (a.ln.gamma && a.ln.residual) return launch<BS, true, true>(a, dsum, st);
-    if (a.ln.gamma) return launch<BS, true, false>(a, dsum, st);
-    return launch<BS, false, false>(a, dsum, st);
+    if (a.normalize) return launch<BS, false, true>(a, dsum, st);
+    if (a.ln.gamma) return launch<BS, true>(a, dsum, st);
+    return launch<BS, false>(a, dsum, st);
 }
 
 }  // namespace
@@ -330,8 +323,7 @@ bool cross_rows_gated_supports(const StepArgs &a) {
     return a.dtype == GRIDNET_F32 && (bs == 4 || bs == 8) && k_ok(a.K) && a.M % bs == 0 && a.N % bs == 0;
 }
 int cross_rows_gated_launch(const StepArgs &a, const float *dsum, hipStream_t st) {
-    return a.block_size == 8 ? launch<8, false, false, false, 2>(a, dsum, st)
-                             : launch<4, false, false, false, 2>(a, dsum, st);
+    return a.block_size == 8 ? launch<8, false, false, 2>(a, dsum, st) : launch<4, false, false, 2>(a, dsum, st);
 }
 
 }  // namespace gridnet

@@ -31,11 +31,11 @@ struct LnFold {
     // when y_raw is null: the last step of a chain) or formed on load as
     // g_prev + LayerNorm'(dy; y_raw, y_stats, y_sums), the gradient with respect to h'' of the
     // step after plus that step's dn taken through its LayerNorm, and then also stored to g_out;
-    // dx receives dn = (gradient with respect to n) - G', and x_part its LayerNorm sums.
+    // dx receives dn = (gradient with respect to n) - G' (the first kernel takes G' off the part
+    // of dx that it writes), and x_part its LayerNorm sums.
     int residual;
     const float *g_prev;  // [B,M,N,K] or null
     float *g_out;         // [B,M,N,K] or null
-    const float *g_rows;  // [B,M,N,K] G' for the cross-block kernel: g_out, or dy when given
     // The backward of a chain (chain_bwd.hip) hands what crosses a block boundary to the backward
     // of the step BEFORE it instead of completing dx itself: per (element, block) the 488
     // values that the cells around the block receive from it, filed per RECEIVING block

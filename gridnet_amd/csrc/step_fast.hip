@@ -302,9 +302,12 @@ void step_fwd_split(
     using FX = Fetch<TL>;
     static_assert(!(NORM && (LN || RES)), "the folded LayerNorm comes without normalisation");
     // two copies of the window; then, for the folded LayerNorm, gamma and beta laid out alike;
-    // for NORM, per wave the four sums taken at commit and, twice, the two of the owned cells
-    __shared__ __attribute__((aligned(16))) float lds[(LN ? 4 : 2) * SW::COPY + (NORM ? 16 : 0)];
+    // for NORM, per wave the four sums taken at commit and, twice, the two of the owned cells;
+    // for RES, twice (alternating between elements) what the owned cells get back at the end:
+    // their raw input minus what the stencil saw of it, laid out like the centre part
+    __shared__ __attribute__((aligned(16))) float lds[(LN ? 4 : 2) * SW::COPY + (NORM ? 16 : 0) + (RES ? 2 * SW::CEN : 0)];
     float *gwin = lds + 2 * SW::COPY, *bwin = gwin + SW::COPY;
+    float *back = lds + 4 * SW::COPY;  // RES (which comes with LN)
     float *sums_at_commit = lds + 2 * SW::COPY, *own_sums = sums_at_commit + 8;  // NORM: [2][4], [2][2][2]
     const int wave = threadIdx.x >> 6;
     const bool ln_in = LN && ln.x_stats != nullptr;  // x is the raw output of the step before
@@ -373,7 +376,8 @@ void step_fwd_split(
     // Fetch::commit_sums; `pre_shift` belongs to `pre`, `shift` to the element being iterated
     float pre_shift = 0.f, shift = 0.f, done_shift = 0.f;
     const int first_cell = (pl.p0 * N + pl.q0) * K + pl.r0;
-    auto commit = [&](float *to, int copies, const typename FX::Buf &v, bool fold, float mean, float rstd) {
+    auto commit = [&](float *to, int copies, const typename FX::Buf &v, bool fold, float mean, float rstd,
+                      float *give_back = nullptr) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) part[q] = 0.f;
 #pragma unroll
@@ -385,10 +389,18 @@ void step_fwd_split(
                 if (LN && fold) {
                     const float4 g4 = *reinterpret_cast<const float4 *>(gwin + cen_at[e]);
                     const float4 b4 = *reinterpret_cast<const float4 *>(bwin + cen_at[e]);
-                    c[0] = fmaf((c[0] - mean) * rstd, g4.x, b4.x);
-                    c[1] = fmaf((c[1] - mean) * rstd, g4.y, b4.y);
-                    c[2] = fmaf((c[2] - mean) * rstd, g4.z, b4.z);
-                    c[3] = fmaf((c[3] - mean) * rstd, g4.w, b4.w);
+                    float n[4];
+                    n[0] = fmaf((c[0] - mean) * rstd, g4.x, b4.x);
+                    n[1] = fmaf((c[1] - mean) * rstd, g4.y, b4.y);
+                    n[2] = fmaf((c[2] - mean) * rstd, g4.z, b4.z);
+                    n[3] = fmaf((c[3] - mean) * rstd, g4.w, b4.w);
+                    // RES: raw minus normalised, for whoever owns these cells (rows of the halo
+                    // leave entries nobody reads)
+                    if (RES && give_back)
+                        *reinterpret_cast<float4 *>(give_back + cen_at[e]) =
+                            make_float4(c[0] - n[0], c[1] - n[1], c[2] - n[2], c[3] - n[3]);
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) c[r] = n[r];
                     end = fmaf((end - mean) * rstd, gwin[side_at[e]], bwin[side_at[e]]);
                 }
                 if (!(fx.ok[e] && fx.edge_ok[e])) end = 0.f;
@@ -450,7 +462,7 @@ void step_fwd_split(
     const bool turns = nchunk > 1;
     for (int s = s0; s < s1; ++s) {
         if (turns) take_turns(s);
-        commit(lds, 2, pre, ln_in, pre_mean, pre_rstd);
+        commit(lds, 2, pre, ln_in, pre_mean, pre_rstd, RES ? back + ((s - s0) & 1) * SW::CEN : nullptr);
         if (NORM) {
             shift = pre_shift;
 #pragma unroll
@@ -462,7 +474,7 @@ void step_fwd_split(
         lds_barrier();
         if (done_s >= 0) store_result(done_s, done);
         if (s + 1 < s1) fetch_element(s + 1);  // next element, in flight
-        float cur[4], base[4], raw[4];
+        float cur[4];
         {
             const float4 q = *reinterpret_cast<const float4 *>(lds + own);
             cur[0] = q.x; cur[1] = q.y; cur[2] = q.z; cur[3] = q.w;
@@ -472,15 +484,6 @@ void step_fwd_split(
             const float4 a4 = *reinterpret_cast<const float4 *>(sums_at_commit);
             const float4 b4 = *reinterpret_cast<const float4 *>(sums_at_commit + 4);
             halo1 = a4.x + b4.x; halo2 = a4.y + b4.y; own1 = a4.z + b4.z; own2 = a4.w + b4.w;
-        }
-        if (RES) {  // the raw input of the owned cells, in register order like `cur`
-            float rt[4];
-            load_cells<4>(x + s * cells + pl.gc, rt);
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                raw[r] = second ? rt[3 - r] : rt[r];
-                base[r] = cur[r];
-            }
         }
         for (int it = 0; it < inner; ++it) {
             const float *from = lds + (it & 1) * SW::COPY;
@@ -531,9 +534,9 @@ void step_fwd_split(
             }
             lds_barrier();
         }
-        if (RES) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) cur[r] = raw[r] + (cur[r] - base[r]);
+        if (RES) {  // x + (result - n): the difference x - n was left at commit, in register order
+            const float4 q = *reinterpret_cast<const float4 *>(back + ((s - s0) & 1) * SW::CEN + own);
+            cur[0] += q.x; cur[1] += q.y; cur[2] += q.z; cur[3] += q.w;
         }
         if (LN && ln.y_part) {
             // statistics of the result for the LayerNorm that follows: every group of 16 lanes
@@ -1260,7 +1263,9 @@ void step_bwd_fast(
         done_s = active ? s : -1;
 #pragma unroll
         for (int c = 0; c < CPT; ++c) {
-            g_done[c] = g[c];
+            // RES: what leaves is dn = (gradient with respect to n) - G'; the cells' own part takes
+            // the whole of G', the cross-block kernel adds the rest of the first term
+            g_done[c] = RES ? g[c] - gin[c] : g[c];
             d_done[c] = dsum[c];
             if (RES) gin_done[c] = gin[c];
         }
@@ -1372,9 +1377,9 @@ void step_bwd_fast(
 // row threads, which hold the finished rows, then also form the two per-sample sums that
 // LayerNorm's backward needs, sum(gamma dx) and sum(gamma dx xhat), and leave them per 16 lanes;
 // for that they load their row of x beside their row of dx.
-// RES (with LN): the outer_residual form of the loop, see LnFold: what is completed here is
-// the gradient with respect to n = LayerNorm(x), and what goes to dx (and into the sums) is
-// dn = that minus G', the gradient with respect to the step's output.
+// RES (with LN): the outer_residual form of the loop, see LnFold: what goes to dx (and into the
+// sums) is dn = (the gradient with respect to n = LayerNorm(x)) - G', G' the gradient with respect
+// to the step's output; step_bwd_fast has taken G' off the cells' own part, so nothing differs here.
 // NORM (per-window normalisation, see step_bwd_fast): `dsum` holds D1, and a cell that lies in
 // the halo of a neighbouring block a additionally receives R_a - x Q_a from it, Q and R being
 // the two numbers per (element, block) that step_bwd_fast left in `qr`.  The row threads add
@@ -1495,7 +1500,6 @@ void step_bwd_cross(
     };
     float gx[E][BS];  // row threads: dx of their row so far (the own block's part)
     float xr[E][BS], xmean[E], xrstd[E];  // LN, row threads: their row of x and its statistics
-    float gr[E][BS];                       // RES, row threads: their row of G'
     int r_prev = -1;
     // the round before: its parts are all in slab `st` by now (a barrier lies in between)
     auto finish_prev = [&](int st) {
@@ -1518,10 +1522,6 @@ void step_bwd_cross(
                     load_cells<BS>(slab + (rj == 0 ? 2 : 3) * FS + ri * BS, part);
 #pragma unroll
                     for (int c = 0; c < BS; ++c) gx[e][c] += part[c];
-                }
-                if (RES) {
-#pragma unroll
-                    for (int c = 0; c < BS; ++c) gx[e][c] -= gr[e][c];
                 }
                 if (NORM) {
                     // neighbours that have this row in their halo, by their offset along K:
@@ -1586,7 +1586,6 @@ void step_bwd_cross(
             for (int e = 0; e < E; ++e) {
                 const int sc = min(sample(r, e), s1 - 1);
                 load_cells<BS>(dx + (long)sc * cells + grow, gx[e]);
-                if (RES) load_cells<BS>(ln.g_rows + (long)sc * cells + grow, gr[e]);
                 if (NORM) load_cells<BS>(x + (long)sc * cells + grow, xr[e]);
                 if (ln_in) {
                     load_cells<BS>(x + (long)sc * cells + grow, xr[e]);
@@ -1819,7 +1818,7 @@ int launch_bwd_ln(const StepArgs &a, hipStream_t st) {
     constexpr int XSLOT = BS == 8 ? kCrossSlots8 : kCrossSlots4;
     constexpr int XE = BS == 8 ? kCrossElems8 : kCrossElems4;
     if (cross_rows_supports(a)) return cross_rows_launch(a, st);  // by whole K-rows
-    hipLaunchKernelGGL((step_bwd_cross<BS, XSLOT, XE, LN, RES, NORM>), dim3(padded_grid(p.nblk, p.nchunk)),
+    hipLaunchKernelGGL((step_bwd_cross<BS, XSLOT, XE, LN, false, NORM>), dim3(padded_grid(p.nblk, p.nchunk)),
                        dim3(6 * BS * BS * XSLOT), 0, st, (const float *)a.weight,
                        (const float *)a.x, (const float *)a.workspace, (float *)a.dx, a.B, a.M, a.N,
                        a.K, p.nblk, p.nchunk, p.chunk_len, a.ln, (const float *)qr);
