@@ -392,7 +392,8 @@ def main():
                 "peak_is": "128 B per clock and CU x 256 CUs x the measured core clock; 16-byte reads go "
                            "beyond it on this part, see measured_read_ceiling"},
         "machine": {"core_clock_ghz_under_load": clock,
-                    "hbm_copy_gb_per_s": ceil.get("copy_gb_per_s")},
+                    "hbm_copy_gb_per_s": ceil.get("copy_gb_per_s"),
+                    "hbm_read_gb_per_s": ceil.get("read_gb_per_s")},
         "binds": what_binds(achieved / HBM_PEAK_GBS, counters.get("valu_busy_pct"), counters.get("lds_busy_frac")),
     }
     if not args.no_cpu_baseline:

@@ -21,7 +21,7 @@ namespace {
 
 enum { GRIDNET_PROBE_FMA = 0, GRIDNET_PROBE_LDS = 1, GRIDNET_PROBE_CLOCK = 2, GRIDNET_PROBE_COPY = 3,
        GRIDNET_PROBE_LDS_B32 = 4, GRIDNET_PROBE_LDS_B64 = 5, GRIDNET_PROBE_LDS_B128 = 6,
-       GRIDNET_PROBE_LDS_2XB64 = 7 };
+       GRIDNET_PROBE_LDS_2XB64 = 7, GRIDNET_PROBE_READ = 8 };
 enum { GRIDNET_OK = 0, GRIDNET_ERR_ARGUMENT = 1, GRIDNET_ERR_LAUNCH = 5 };
 
 char *probe_error() {
@@ -147,6 +147,18 @@ __global__ __launch_bounds__(kProbeThreads) void probe_copy(const float4 *src, f
     }
 }
 
+// the same requests, nothing written but one value per thread: what reads alone get from HBM
+// (a kernel that reads more than it writes sits between this figure and the copy's)
+__global__ __launch_bounds__(kProbeThreads) void probe_read(const float4 *src, float *out, size_t n) {
+    const size_t stride = (size_t)gridDim.x * kProbeThreads;
+    float acc = 0.f;
+    for (size_t i = (size_t)blockIdx.x * kProbeThreads + threadIdx.x; i + 3 * stride < n; i += 4 * stride) {
+        const float4 a = src[i], b = src[i + stride], c = src[i + 2 * stride], d = src[i + 3 * stride];
+        acc += (a.x + a.y + a.z + a.w) + (b.x + b.y + b.z + b.w) + (c.x + c.y + c.z + c.w) + (d.x + d.y + d.z + d.w);
+    }
+    out[(size_t)blockIdx.x * kProbeThreads + threadIdx.x] = acc;
+}
+
 struct Timer {
     hipEvent_t e0 = nullptr, e1 = nullptr;
     bool ok;
@@ -226,6 +238,18 @@ extern "C" int gridnet_probe(int what, double *result) {
         hipLaunchKernelGGL(probe_copy, dim3(cus * 32), dim3(kProbeThreads), 0, 0, dst, src, n);  // first touch
         s = timer.best(4, [&] { hipLaunchKernelGGL(probe_copy, dim3(cus * 32), dim3(kProbeThreads), 0, 0, src, dst, n); });
         if (s > 0) *result = 2.0 * (double)n * sizeof(float4) / s / 1e9;
+        break;
+    }
+    case GRIDNET_PROBE_READ: {  // GB/s, reads only
+        const size_t n = (size_t)1 << 26;  // 1 GiB
+        if (hipMalloc(&src, n * sizeof(float4)) != hipSuccess ||
+            hipMalloc(&dst, (size_t)cus * 32 * kProbeThreads * sizeof(float)) != hipSuccess) {
+            rc = fail(GRIDNET_ERR_LAUNCH, "probe: hipMalloc failed");
+            break;
+        }
+        if (hipMemset(src, 0, n * sizeof(float4)) != hipSuccess) { rc = fail(GRIDNET_ERR_LAUNCH, "probe: hipMemset failed"); break; }
+        s = timer.best(4, [&] { hipLaunchKernelGGL(probe_read, dim3(cus * 32), dim3(kProbeThreads), 0, 0, src, (float *)dst, n); });
+        if (s > 0) *result = (double)n * sizeof(float4) / s / 1e9;
         break;
     }
     case GRIDNET_PROBE_LDS_B32:

@@ -1,5 +1,5 @@
 """ctypes binding of libgridnet_probe.so: machine ceilings that bench.py quotes beside the vendor
-peaks (sustained fp32 FMA rate, LDS read rate, core clock under load, an HBM copy, LDS-pipe cycles
+peaks (sustained fp32 FMA rate, LDS read rate, core clock under load, an HBM copy and HBM reads alone, LDS-pipe cycles
 per read width), measured with the kernels' own compiler flags.  Not part of the update path and
 not part of libgridnet_hip.so: it allocates its own buffers, runs on the null stream and
 synchronises."""
@@ -10,7 +10,7 @@ import os
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libgridnet_probe.so")
 
-PROBES = {"fma_tfma_per_s": 0, "lds_gb_per_s": 1, "clock_ghz": 2, "copy_gb_per_s": 3}
+PROBES = {"fma_tfma_per_s": 0, "lds_gb_per_s": 1, "clock_ghz": 2, "copy_gb_per_s": 3, "read_gb_per_s": 8}
 # LDS-pipe cycles per wave-level read instruction, by width
 LDS_WIDTH_PROBES = {"ds_read_b32": 4, "ds_read_b64": 5, "ds_read_b128": 6, "ds_read2_b64": 7}
 

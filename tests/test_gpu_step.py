@@ -265,6 +265,9 @@ def test_machine_ceiling_probes_report_sane_figures():
     assert 1.0e4 < lds < 4.0e5
     assert 0.5 < clock < 3.5
     assert 500.0 < copy < 8000.0    # read + write against 8 TB/s
+    read = p.probe("read_gb_per_s")
+    print(f"        reads alone {read:.0f} GB/s", flush=True)
+    assert 500.0 < read < 8000.0
     widths = {k: p.probe(k) for k in p.LDS_WIDTH_PROBES}
     print("LDS pipe cycles per wave-level read:", {k: round(v, 2) for k, v in widths.items()}, flush=True)
     assert all(1.0 < v < 64.0 for v in widths.values())
