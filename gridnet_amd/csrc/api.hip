@@ -100,7 +100,7 @@ using namespace gridnet;
 
 extern "C" {
 
-int gridnet_hip_version(void) { return 7; }  // 2: fused body; 3: residual forward and backward; 4: gated backward takes a workspace; 5: backward on static scratch; 6: chain backward, gradient copies for split batches; 7: whole chain in one launch
+int gridnet_hip_version(void) { return 8; }  // 2: fused body; 3: residual forward and backward; 4: gated backward takes a workspace; 5: backward on static scratch; 6: chain backward, gradient copies for split batches; 7: whole chain in one launch; 8: fused forward with flags
 
 const char *gridnet_hip_last_error(void) { return error_buffer(); }
 
@@ -351,7 +351,7 @@ static int fused_forward(int dtype, const void *weight, const void *bias, const 
                          const void *gamma, const void *beta, const void *x, const void *x_stats,
                          void *y_raw, void *y_stats, int B, int M, int N, int K, int inner,
                          int block_size, double ln_eps, int activation, void *workspace,
-                         size_t workspace_bytes, void *stream, int residual) {
+                         size_t workspace_bytes, void *stream, int residual, int walk_reverse = 0) {
     StepArgs a{};
     a.dtype = dtype; a.weight = weight; a.bias = bias; a.scale = scale; a.x = x; a.y = y_raw;
     a.B = B; a.M = M; a.N = N; a.K = K; a.inner = inner; a.block_size = block_size;
@@ -371,6 +371,7 @@ static int fused_forward(int dtype, const void *weight, const void *bias, const 
     a.ln.x_stats = (const float *)x_stats;
     a.ln.y_part = (float *)workspace;
     a.ln.residual = residual;
+    a.ln.walk_reverse = walk_reverse;
     if (int rc = step_forward_fast(a, st)) return rc;
     const int nblk = (M / block_size) * (N / block_size) * (K / block_size);
     return layernorm_finalize_stats((const float *)workspace, nblk * step_fast_forward_parts(block_size),
@@ -385,6 +386,18 @@ int gridnet_hip_fused_forward(int dtype, const void *weight, const void *bias, c
                               void *workspace, size_t workspace_bytes, void *stream) {
     return fused_forward(dtype, weight, bias, scale, gamma, beta, x, x_stats, y_raw, y_stats, B, M, N,
                          K, inner, block_size, ln_eps, activation, workspace, workspace_bytes, stream, 0);
+}
+
+int gridnet_hip_fused_forward_flags(int dtype, const void *weight, const void *bias, const void *scale,
+                                    const void *gamma, const void *beta, const void *x,
+                                    const void *x_stats, void *y, void *y_stats, int B, int M, int N,
+                                    int K, int inner, int block_size, double ln_eps, int activation,
+                                    int flags, void *workspace, size_t workspace_bytes, void *stream) {
+    if (flags & ~(GRIDNET_FUSED_RESIDUAL | GRIDNET_FUSED_WALK_REVERSE))
+        return fail(GRIDNET_ERR_ARGUMENT, "unknown flag bits: %d", flags);
+    return fused_forward(dtype, weight, bias, scale, gamma, beta, x, x_stats, y, y_stats, B, M, N, K, inner,
+                         block_size, ln_eps, activation, workspace, workspace_bytes, stream,
+                         (flags & GRIDNET_FUSED_RESIDUAL) ? 1 : 0, (flags & GRIDNET_FUSED_WALK_REVERSE) ? 1 : 0);
 }
 
 int gridnet_hip_fused_forward_residual(int dtype, const void *weight, const void *bias,

@@ -160,6 +160,12 @@ constexpr int kXcds = 8;
 __host__ __device__ __forceinline__ int padded_grid(int nblk, int nchunk) {
     return kXcds * ((nblk + kXcds - 1) / kXcds) * nchunk;
 }
+// The workgroup that takes this one's place when a launch walks its blocks backwards: same XCD
+// (what a block's workgroups left in that XCD's L2 in the launch before stays where it is looked
+// for), the XCD's workgroups in reverse order.  `grid` is a padded_grid().
+__device__ __forceinline__ int reversed_on_its_xcd(int wg, int grid) {
+    return wg % kXcds + kXcds * (grid / kXcds - 1 - wg / kXcds);
+}
 __device__ __forceinline__ bool split_block_id(int wg, int nblk, int nchunk, int &blk, int &chunk) {
     const int per_xcd = (nblk + kXcds - 1) / kXcds;
     const int xcd = wg % kXcds, slot = wg / kXcds;

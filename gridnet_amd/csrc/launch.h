@@ -43,6 +43,10 @@ struct LnFold {
     // dy is complete); halo_out: where this step leaves its own (null: dx is completed here).
     const float *halo_in;
     float *halo_out;
+    // forward: workgroups take the blocks in reverse order.  Results do not depend on it; a chain
+    // whose steps alternate finds what the step before touched last (its output, the parameter
+    // planes it fetched last) still in the last-level cache when its working set exceeds that cache.
+    int walk_reverse;
 };
 
 struct StepArgs {

@@ -81,7 +81,9 @@ void step_fwd_fast(
     static_assert(!(NORM && (LN || RES)), "the folded LayerNorm comes without normalisation");
 
     int blk, chunk;
-    if (!split_block_id(blockIdx.x, nblk, nchunk, blk, chunk)) return;  // grid padding
+    if (!split_block_id(ln.walk_reverse ? reversed_on_its_xcd(blockIdx.x, gridDim.x) : blockIdx.x, nblk, nchunk,
+                        blk, chunk))
+        return;  // grid padding
     const Place<TL, CPT, NSLOT> pl(threadIdx.x, blk, N, K);
     const Fetch<TL> fx(pl.lane, pl.p0, pl.q0, pl.r0, M, N, K);
     float *win = lds + pl.slot * (2 * TL::WIN);
@@ -313,7 +315,9 @@ void step_fwd_split(
     const bool ln_in = LN && ln.x_stats != nullptr;  // x is the raw output of the step before
 
     int blk, chunk;
-    if (!split_block_id(blockIdx.x, nblk, nchunk, blk, chunk)) return;  // grid padding
+    if (!split_block_id(ln.walk_reverse ? reversed_on_its_xcd(blockIdx.x, gridDim.x) : blockIdx.x, nblk, nchunk,
+                        blk, chunk))
+        return;  // grid padding
     const Place<TL, 4, 1> pl(threadIdx.x, blk, N, K);
     const FX fx(pl.lane, pl.p0, pl.q0, pl.r0, M, N, K);
     const long cells = (long)M * N * K;
@@ -592,7 +596,9 @@ void step_fwd_pair(
     const bool ln_in = ln.x_stats != nullptr;  // x is the raw output of the step before
 
     int blk, chunk;
-    if (!split_block_id(blockIdx.x, nblk, nchunk, blk, chunk)) return;  // grid padding
+    if (!split_block_id(ln.walk_reverse ? reversed_on_its_xcd(blockIdx.x, gridDim.x) : blockIdx.x, nblk, nchunk,
+                        blk, chunk))
+        return;  // grid padding
     const Place<TL, 4, 1> pl(threadIdx.x, blk, N, K);
     const FX fx(pl.lane, pl.p0, pl.q0, pl.r0, M, N, K);
     const long cells = (long)M * N * K;

@@ -16,6 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("GRIDNET_HIP_LIBRARY") or os.path.join(_HERE, "libgridnet_hip.so")
 
 F32, F64 = 0, 1
+FUSED_RESIDUAL, FUSED_WALK_REVERSE = 1, 2  # gridnet_hip_fused_forward_flags
 OVERWRITE_PARAMS = 1
 OVERWRITE_DX = 2
 OVERWRITE = 3
@@ -39,6 +40,7 @@ EXPORTS = (
     "gridnet_hip_fused_workspace_bytes",
     "gridnet_hip_fused_forward",
     "gridnet_hip_fused_forward_residual",
+    "gridnet_hip_fused_forward_flags",
     "gridnet_hip_layernorm_apply",
     "gridnet_hip_layernorm_backward_sums",
     "gridnet_hip_fused_backward",
@@ -98,6 +100,9 @@ def _load():
     lib.gridnet_hip_fused_forward.restype = i
     lib.gridnet_hip_fused_forward.argtypes = [i, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, d, i,
                                               p, z, p]
+    lib.gridnet_hip_fused_forward_flags.restype = i
+    lib.gridnet_hip_fused_forward_flags.argtypes = [i, p, p, p, p, p, p, p, p, p, i, i, i, i, i, i, d, i, i,
+                                                    p, z, p]
     lib.gridnet_hip_fused_forward_residual.restype = i
     lib.gridnet_hip_fused_forward_residual.argtypes = lib.gridnet_hip_fused_forward.argtypes
     lib.gridnet_hip_layernorm_apply.restype = i

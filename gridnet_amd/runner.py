@@ -194,12 +194,16 @@ class BodyRunner:
             y = self.s[j] if keep else (self.s[0], self.h[1])[j % 2]
             y_stats = self.stats[j if keep else j % 2]
             self._mark("step_fwd", 0)
-            _n.check(_n.lib.gridnet_hip_fused_forward(
+            # every other step walks the blocks in reverse: what the step before touched last is
+            # what this one needs first (it matters where a step's working set exceeds the
+            # last-level cache, a 128^3 grid; the results are the same bits)
+            _n.check(_n.lib.gridnet_hip_fused_forward_flags(
                 self.dt, *self._params(j),
                 self.gamma.data_ptr(), self.beta.data_ptr(), x.data_ptr(),
                 x_stats.data_ptr() if x_stats is not None else None, y.data_ptr(),
                 y_stats.data_ptr(), self.B, self.M, self.N, self.K, self.inner, self.bs,
-                self.ln_eps, self.act, self.fw_ws.data_ptr(), self.fw_ws_bytes, stream))
+                self.ln_eps, self.act, _n.FUSED_WALK_REVERSE if j & 1 else 0,
+                self.fw_ws.data_ptr(), self.fw_ws_bytes, stream))
             self._mark("step_fwd", 1)
             x, x_stats = y, y_stats
         out = self.h[0]
@@ -225,11 +229,13 @@ class BodyRunner:
             out = self.h[j + 1] if keep else (self.s[0], self.h[1])[j % 2]
             out_stats = self.stats[j + 1 if keep else (j + 1) % 2]
             self._mark("step_fwd", 0)
-            _n.check(_n.lib.gridnet_hip_fused_forward_residual(
+            _n.check(_n.lib.gridnet_hip_fused_forward_flags(
                 self.dt, *self._params(j),
                 self.gamma.data_ptr(), self.beta.data_ptr(), h.data_ptr(), stats.data_ptr(),
                 out.data_ptr(), out_stats.data_ptr(), self.B, self.M, self.N, self.K, self.inner,
-                self.bs, self.ln_eps, self.act, self.fw_ws.data_ptr(), self.fw_ws_bytes, stream))
+                self.bs, self.ln_eps, self.act,
+                _n.FUSED_RESIDUAL | (_n.FUSED_WALK_REVERSE if j & 1 else 0),
+                self.fw_ws.data_ptr(), self.fw_ws_bytes, stream))
             self._mark("step_fwd", 1)
             h, stats = out, out_stats
         return h

@@ -206,6 +206,21 @@ int gridnet_hip_fused_forward(int dtype, const void *weight, const void *bias, c
                               int K, int inner, int block_size, double ln_eps, int activation,
                               void *workspace, size_t workspace_bytes, void *stream);
 
+/* Either of the two forward calls around this one (gridnet_hip_fused_forward,
+ * gridnet_hip_fused_forward_residual with GRIDNET_FUSED_RESIDUAL) with one more choice:
+ * GRIDNET_FUSED_WALK_REVERSE makes the workgroups take the blocks in reverse order.  The results
+ * are the same bits either way.  A chain of steps (gridnet/scripts/train_imagenet.py:76-86) that
+ * sets it for every other step finds what the step before touched last -- the end of its output,
+ * the parameter planes it fetched last -- still in the GPU's last-level cache when one step's
+ * working set exceeds that cache (a 128^3 grid: 243 MB of parameters per step against 256 MB of
+ * cache; 162 -> 156 us per step there, nothing to gain at 64^3). */
+enum { GRIDNET_FUSED_RESIDUAL = 1, GRIDNET_FUSED_WALK_REVERSE = 2 };
+int gridnet_hip_fused_forward_flags(int dtype, const void *weight, const void *bias, const void *scale,
+                                    const void *gamma, const void *beta, const void *x,
+                                    const void *x_stats, void *y, void *y_stats, int B, int M, int N,
+                                    int K, int inner, int block_size, double ln_eps, int activation,
+                                    int flags, void *workspace, size_t workspace_bytes, void *stream);
+
 /* The reference's outer_residual form of one outer step, forward
  * (gridnet/scripts/train_imagenet.py:81-83: n = norm(h); h = h + (net(n) - n)):
  * y = x + (step(n) - n) with n = LayerNorm(x; x_stats, gamma, beta), y_stats = statistics of y,

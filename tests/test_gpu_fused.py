@@ -335,3 +335,41 @@ def test_fused_rejects_what_it_does_not_cover():
     rc = n.lib.gridnet_hip_fused_forward(n.F32, p, p, p, p, p, p, None, p, p, 1, 8, 8, 8, 1, 8, 1e-5,
                                          0, p, 0, n.current_stream(x))
     assert rc != 0 and "workspace" in n.last_error()
+
+
+@pytest.mark.parametrize("bs,shape,batch", [(8, (16, 32, 16), 5), (4, (8, 8, 16), 3), (8, (16, 16, 16), 20)])
+def test_fused_forward_flags_match_the_plain_entry_points(bs, shape, batch):
+    """gridnet_hip_fused_forward_flags: with no flag and with GRIDNET_FUSED_RESIDUAL it is the two
+    forward entry points beside it, and the order in which the workgroups take the blocks
+    (GRIDNET_FUSED_WALK_REVERSE) changes no bit of the results; unknown flag bits are refused."""
+    from gridnet_amd import native as n
+    from helpers import make_acts, make_params
+
+    print(f"fused forward flags bs={bs} shape={shape} batch={batch}", flush=True)
+    w, b, r = (v.to(DEV) for v in make_params(shape, seed=41))
+    g = torch.Generator().manual_seed(42)
+    gamma = (1 + 0.2 * torch.randn(shape, generator=g)).to(DEV)
+    beta = (0.2 * torch.randn(shape, generator=g)).to(DEV)
+    x = make_acts(batch, shape, seed=43).to(DEV)
+    flat = x.flatten(1)
+    stats = torch.stack([flat.mean(1), 1 / torch.sqrt(flat.var(1, unbiased=False) + 1e-5)], 1).contiguous()
+    M, N, K = shape
+    ws_bytes = n.lib.gridnet_hip_fused_workspace_bytes(batch, M, N, K, 3, bs, 0)
+    ws = n.workspace(ws_bytes, x.device)
+    stream = n.current_stream(x)
+    act = n.activation_id("silu")
+
+    def call(fn, *flags):
+        y, ys = torch.full_like(x, float("nan")), torch.empty(batch, 2, device=DEV)
+        n.check(fn(n.dtype_id(x), w.data_ptr(), b.data_ptr(), r.data_ptr(), gamma.data_ptr(), beta.data_ptr(),
+                   x.data_ptr(), stats.data_ptr(), y.data_ptr(), ys.data_ptr(), batch, M, N, K, 3, bs, 1e-5, act,
+                   *flags, ws.data_ptr(), ws_bytes, stream))
+        return y, ys
+
+    for base, flag in ((n.lib.gridnet_hip_fused_forward, 0), (n.lib.gridnet_hip_fused_forward_residual, n.FUSED_RESIDUAL)):
+        want = call(base)
+        for extra in (0, n.FUSED_WALK_REVERSE):
+            got = call(n.lib.gridnet_hip_fused_forward_flags, flag | extra)
+            assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1]), (flag, extra)
+    with pytest.raises(RuntimeError, match="flag"):
+        call(n.lib.gridnet_hip_fused_forward_flags, 4)
