@@ -79,6 +79,9 @@ WORKLOADS = {
     # C3 with the inner iteration count of the reference's own ImageNet script
     # (gridnet/scripts/train_imagenet.py:101-104: inner 8, outer 12, grid 64, batch 32)
     "C3i8": Workload("C3i8 64^3 bs8 B32 inner8 outer12 fwd+bwd", 64, 8, 32, 8, 12, True),
+    # the defaults of the reference's MNIST script (gridnet/scripts/train_mnist.py:45-53, 74-78):
+    # 32^3 grid, 8^3 blocks, batch 256, one inner iteration, 64 outer steps, silu, training
+    "M": Workload("M 32^3 bs8 B256 inner1 outer64 fwd+bwd silu", 32, 8, 256, 1, 64, True, activation="silu"),
 }
 
 
