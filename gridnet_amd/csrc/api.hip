@@ -373,10 +373,8 @@ static int fused_forward(int dtype, const void *weight, const void *bias, const 
     a.ln.residual = residual;
     a.ln.walk_reverse = walk_reverse;
     if (int rc = step_forward_fast(a, st)) return rc;
-    const int nblk = (M / block_size) * (N / block_size) * (K / block_size);
-    return layernorm_finalize_stats((const float *)workspace, nblk * step_fast_forward_parts(block_size),
-                                    step_fast_forward_part_count(block_size), (float *)y_stats, B,
-                                    ln_eps, st);
+    return layernorm_finalize_stats((const float *)workspace, step_fast_forward_pairs(a),
+                                    step_fast_forward_pair_count(a), (float *)y_stats, B, ln_eps, st);
 }
 
 int gridnet_hip_fused_forward(int dtype, const void *weight, const void *bias, const void *scale,

@@ -42,14 +42,6 @@ template <int BS> struct Tube {
     static_assert(BS == 4 || BS == 8, "block sizes 4 and 8");
 };
 
-// the lane before / after in the wave (the caller masks the ends of a row)
-__device__ __forceinline__ float lane_before(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x138, 0xf, 0xf, false));
-}
-__device__ __forceinline__ float lane_after(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x130, 0xf, 0xf, false));
-}
-
 template <int BS, bool LN, bool NORM = false, int SETS = 1>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(SETS == 1 ? 3 : 2, SETS == 1 ? 3 : 2)))
 void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,

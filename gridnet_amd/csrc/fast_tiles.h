@@ -84,6 +84,15 @@ __device__ __forceinline__ float row16_sum(float v) {
     return v;
 }
 
+// The value of `v` in the lane before / after the caller's in the wave (DPP wave shifts: no LDS
+// access).  For kernels whose lanes run along a grid row: the caller masks the ends of its row.
+__device__ __forceinline__ float lane_before(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x138, 0xf, 0xf, false));
+}
+__device__ __forceinline__ float lane_after(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x130, 0xf, 0xf, false));
+}
+
 // Sum of `v` over those lanes of the calling wave that belong to the caller's slot: the whole
 // wave for slots of 64 threads and more, the caller's half of it for 32-thread slots.  Row
 // rotations, then the four row totals are read across as scalars: no LDS, and every lane of the

@@ -103,10 +103,18 @@ size_t step_fast_slab_bytes(const StepArgs &a);           // room for the gradie
 int step_forward_fast(const StepArgs &a, hipStream_t st);
 int step_backward_fast(const StepArgs &a, hipStream_t st);
 // partial statistics per (block, batch element) that the kernels above write when asked to
-int step_fast_forward_parts(int block_size);   // (mean, M2) pairs, each over forward_part_count cells
+int step_fast_forward_parts(int block_size);   // (mean, M2) pairs per block at most, each over forward_part_count cells
 int step_fast_forward_part_count(int block_size);
+int step_fast_forward_pairs(const StepArgs &a);       // pairs per sample that the forward of `a` leaves ...
+int step_fast_forward_pair_count(const StepArgs &a);  // ... and the cells behind each
 int step_fast_backward_parts(int block_size);  // (sum g, sum g*xhat) pairs per (block, element), at most
 int step_fast_backward_pairs(const StepArgs &a);  // pairs per sample that the backward of `a` leaves
+
+// fwd_rows.hip: the forward of a step with ONE inner iteration, dealt by whole K-rows (fp32, normalize
+// off, K of 16, 32, 64 or 128; the folded LayerNorm and the residual form as a.ln says)
+bool fwd_rows_supports(const StepArgs &a);
+int fwd_rows_pairs(const StepArgs &a);  // (mean, M2) pairs per sample in a.ln.y_part, 256 cells each
+int fwd_rows_launch(const StepArgs &a, hipStream_t st);
 
 // cross_rows.hip: the cross-block part of the backward for 4^3 blocks, dealt by whole K-rows
 // (a.workspace holds D, a.dx the block-local part; LayerNorm fold as a.ln says); K of 16, 32, 64

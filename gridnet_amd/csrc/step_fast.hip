@@ -1907,6 +1907,13 @@ int step_fast_forward_part_count(int block_size) {
 }
 // per block at most: the kernel dealt by block face leaves one pair per block, the row-wise one a
 // pair per 256 cells (two per 8^3 block, a quarter per 4^3 block)
+int step_fast_forward_pairs(const StepArgs &a) {
+    if (fwd_rows_supports(a)) return fwd_rows_pairs(a);
+    return (a.M / a.block_size) * (a.N / a.block_size) * (a.K / a.block_size) * step_fast_forward_parts(a.block_size);
+}
+int step_fast_forward_pair_count(const StepArgs &a) {
+    return fwd_rows_supports(a) ? 256 : step_fast_forward_part_count(a.block_size);
+}
 int step_fast_backward_parts(int block_size) { return block_size == 8 ? 2 : 1; }
 int step_fast_backward_pairs(const StepArgs &a) {
     if (cross_rows_supports(a)) return cross_rows_pairs(a);
@@ -1947,7 +1954,10 @@ size_t step_fast_slab_bytes(const StepArgs &a) {
     return (size_t)chunks * kStepSlabPlanes * a.M * a.N * a.K * sizeof(float);
 }
 
-int step_forward_fast(const StepArgs &a, hipStream_t st) { return dispatch<false>(a, st); }
+int step_forward_fast(const StepArgs &a, hipStream_t st) {
+    if (fwd_rows_supports(a)) return fwd_rows_launch(a, st);  // one inner iteration: a plain stencil, by whole rows
+    return dispatch<false>(a, st);
+}
 int step_backward_fast(const StepArgs &a, hipStream_t st) { return dispatch<true>(a, st); }
 
 }  // namespace gridnet

@@ -78,6 +78,12 @@ MATRIX = [
     ((8, 12, 64), 4, 3, True, "tanh"),
     ((16, 8, 32), 8, 2, True, "silu"),
     ((8, 4, 16), 4, 2, True, "relu"),
+    # one inner iteration with rows of 16, 32, 64 and 128 cells: the forward is a plain stencil there
+    # and goes by whole rows (csrc/fwd_rows.hip), whatever the block size
+    ((8, 12, 16), 4, 1, False, "silu"),
+    ((16, 8, 32), 8, 1, False, "tanh"),
+    ((8, 16, 64), 8, 1, False, "leaky_relu"),
+    ((4, 8, 128), 4, 1, False, "relu"),
     # no inner iteration on a grid of several blocks: the gradient passes through unchanged
     ((16, 24, 16), 8, 0, True, "silu"),
     ((8, 16, 8), 4, 0, False, "tanh"),
