@@ -12,7 +12,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libgridnet_hip.so")
-SOURCES = ["api.hip", "step_generic.hip", "step_fast.hip", "fwd_rows.hip", "cross_rows.hip", "chain_bwd.hip", "gated_generic.hip", "gated_fast.hip", "layernorm.hip"]
+SOURCES = ["api.hip", "step_generic.hip", "step_fast.hip", "fwd_rows.hip", "bwd_rows.hip", "cross_rows.hip", "chain_bwd.hip", "gated_generic.hip", "gated_fast.hip", "layernorm.hip"]
 # machine ceilings for bench.py: not part of the product library (it allocates and synchronises)
 PROBE_LIB = os.path.join(HERE, "libgridnet_probe.so")
 PROBE_SOURCES = ["probe.hip"]

@@ -42,7 +42,10 @@ template <int BS> struct Tube {
     static_assert(BS == 4 || BS == 8, "block sizes 4 and 8");
 };
 
-template <int BS, bool LN, bool NORM = false, int SETS = 1>
+// FULL: ALL taps, not only those that leave the block: the second kernel of the backward of a step
+// with one inner iteration (bwd_rows.hip), where `dsum` holds delta of every cell and dx the
+// direct part of the gradient.
+template <int BS, bool LN, bool NORM = false, int SETS = 1, bool FULL = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(SETS == 1 ? 3 : 2, SETS == 1 ? 3 : 2)))
 void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
                 const float *__restrict__ dsum, float *__restrict__ dx, int B, int M, int N, int K,
@@ -72,21 +75,30 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
         const int gi = p0 + ci + di, gj = q0 + cj + dj;
         const bool side = bi + di < 0 || bi + di >= BS || bj + dj < 0 || bj + dj >= BS;
         const bool row_ok = gi >= 0 && gi < M && gj >= 0 && gj < N;
+        // A tap's four weights W[26-t, h] for the thread's cells lie side by side along K, one
+        // cell off its own four for dk = -1 / +1: one aligned 16-byte load per tap (every lane of
+        // the row loads its own piece of the same plane and row) and the missing end from the lane
+        // next door, instead of four scattered 4-byte loads.
+        const int rowbase = row_ok ? (gi * N + gj) * K + 4 * bk : grow;
 #pragma unroll
-        for (int dk = -1; dk <= 1; ++dk)
+        for (int k = 0; k < SETS; ++k)
 #pragma unroll
-            for (int ck = 0; ck < 4; ++ck) {
-                // a tap along K can only cross where it leaves the thread's four cells (known
-                // when compiling); taps that never cross are not held at all
-                if (pq == 4 && !(ck + dk < 0 || ck + dk > 3)) continue;
-                const bool along = bk0 + ck + dk < 0 || bk0 + ck + dk >= BS;
-                const int gk = 4 * bk + ck + dk;
+            for (int dk = -1; dk <= 1; ++dk) {
                 const int t = (di + 1) * 9 + (dj + 1) * 3 + (dk + 1);
-                const bool use = (side || along) && row_ok && gk >= 0 && gk < K;
-                const long h = ((long)gi * N + gj) * K + gk;
+                float piece[4];
+                load_cells<4>(weight + ((26 - t) * SETS + k) * cells + rowbase, piece);
+                const float before = lane_before(piece[3]), after = lane_after(piece[0]);
 #pragma unroll
-                for (int k = 0; k < SETS; ++k)
-                    vx[k][pq][dk + 1][ck] = use ? weight[((26 - t) * SETS + k) * cells + h] : 0.f;
+                for (int ck = 0; ck < 4; ++ck) {
+                    // a tap along K can only cross where it leaves the thread's four cells (known
+                    // when compiling); taps that never cross are not held at all
+                    if (!FULL && pq == 4 && !(ck + dk < 0 || ck + dk > 3)) continue;
+                    const bool along = bk0 + ck + dk < 0 || bk0 + ck + dk >= BS;
+                    const int gk = 4 * bk + ck + dk;
+                    const bool use = (FULL || side || along) && row_ok && gk >= 0 && gk < K;
+                    const float wv = ck + dk < 0 ? before : ck + dk > 3 ? after : piece[(ck + dk) & 3];
+                    vx[k][pq][dk + 1][ck] = use ? wv : 0.f;
+                }
             }
     }
     const bool ln_in = LN && ln.x_stats != nullptr;
@@ -198,7 +210,7 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
             for (int dk = -1; dk <= 1; ++dk)
 #pragma unroll
                 for (int ck = 0; ck < 4; ++ck) {
-                    if (pq == 4 && !(ck + dk < 0 || ck + dk > 3)) continue;
+                    if (!FULL && pq == 4 && !(ck + dk < 0 || ck + dk > 3)) continue;
                     g[ck] = fmaf(vx[k][pq][dk + 1][ck], d[ck + 1 + dk], g[ck]);
                 }
         }
@@ -251,10 +263,10 @@ void cross_rows(const float *__restrict__ weight, const float *__restrict__ x,
 
 bool k_ok(int K) { return K == 16 || K == 32 || K == 64 || K == 128; }
 
-template <int BS, bool LN, bool NORM = false, int SETS = 1>
+template <int BS, bool LN, bool NORM = false, int SETS = 1, bool FULL = false>
 int launch(const StepArgs &a, const float *dsum, hipStream_t st) {
     using TB = Tube<BS>;
-    auto kern = cross_rows<BS, LN, NORM, SETS>;
+    auto kern = cross_rows<BS, LN, NORM, SETS, FULL>;
     const int nt = 4 * a.K, ntube = (a.M / TB::RI) * (a.N / TB::RJ);
     const size_t lds = ((size_t)2 * SETS * TB::ROWS * a.K + (NORM ? 2 * 9 * (a.K / BS + 2) * 2 : 0)) * sizeof(float);
     static bool big_lds_enabled = false;  // per instantiation
@@ -307,6 +319,12 @@ int cross_rows_pairs(const StepArgs &a) { return (a.M * a.N / 16) * (4 * a.K / 6
 
 int cross_rows_launch(const StepArgs &a, hipStream_t st) {
     return a.block_size == 8 ? dispatch<8>(a, st) : dispatch<4>(a, st);
+}
+
+// all 27 taps (the second kernel of bwd_rows.hip); the block size does not enter then
+int cross_rows_full_launch(const StepArgs &a, hipStream_t st) {
+    const float *dsum = (const float *)a.workspace;
+    return a.ln.gamma ? launch<4, true, false, 1, true>(a, dsum, st) : launch<4, false, false, 1, true>(a, dsum, st);
 }
 
 // the gated update: weight [27, 2, M, N, K], D0 and D1 of every cell behind one another in `dsum`

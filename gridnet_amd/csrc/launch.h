@@ -116,12 +116,20 @@ bool fwd_rows_supports(const StepArgs &a);
 int fwd_rows_pairs(const StepArgs &a);  // (mean, M2) pairs per sample in a.ln.y_part, 256 cells each
 int fwd_rows_launch(const StepArgs &a, hipStream_t st);
 
+// bwd_rows.hip: the backward of a step with ONE inner iteration by whole K-rows (with
+// cross_rows_full_launch behind it); fp32, normalize off, K of 16, 32 or 64; a.slabs as for
+// step_backward_fast
+bool bwd_rows_supports(const StepArgs &a);
+size_t bwd_rows_slab_bytes(const StepArgs &a);
+int bwd_rows_launch(const StepArgs &a, hipStream_t st);
+
 // cross_rows.hip: the cross-block part of the backward for 4^3 blocks, dealt by whole K-rows
 // (a.workspace holds D, a.dx the block-local part; LayerNorm fold as a.ln says); K of 16, 32, 64
 // or 128, normalize off
 bool cross_rows_supports(const StepArgs &a);
 int cross_rows_pairs(const StepArgs &a);  // LayerNorm sum pairs per sample that it leaves in a.ln.x_part
 int cross_rows_launch(const StepArgs &a, hipStream_t st);
+int cross_rows_full_launch(const StepArgs &a, hipStream_t st);  // all 27 taps, for bwd_rows.hip
 bool cross_rows_gated_supports(const StepArgs &a);  // the gated update: two weight sets, D0 and D1 in `dsum`
 int cross_rows_gated_launch(const StepArgs &a, const float *dsum, hipStream_t st);
 

@@ -1942,6 +1942,7 @@ size_t step_fast_backward_workspace(const StepArgs &a) {
 }
 
 size_t step_fast_slab_bytes(const StepArgs &a) {
+    if (bwd_rows_supports(a)) return bwd_rows_slab_bytes(a);
     // the most chunks any plan of the backward kernels makes: resident workgroups (two per CU with
     // 8^3 blocks, bounded by 16 with 4^3) over the blocks, and never more than the batch gives
     const long nblk = (long)(a.M / a.block_size) * (a.N / a.block_size) * (a.K / a.block_size);
@@ -1958,6 +1959,9 @@ int step_forward_fast(const StepArgs &a, hipStream_t st) {
     if (fwd_rows_supports(a)) return fwd_rows_launch(a, st);  // one inner iteration: a plain stencil, by whole rows
     return dispatch<false>(a, st);
 }
-int step_backward_fast(const StepArgs &a, hipStream_t st) { return dispatch<true>(a, st); }
+int step_backward_fast(const StepArgs &a, hipStream_t st) {
+    if (bwd_rows_supports(a)) return bwd_rows_launch(a, st);  // one inner iteration: by whole rows
+    return dispatch<true>(a, st);
+}
 
 }  // namespace gridnet
