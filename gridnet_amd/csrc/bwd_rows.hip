@@ -99,6 +99,11 @@ void bwd_rows(const float *__restrict__ weight, const float *__restrict__ bias, 
             float gq[4], bq[4];
             load_cells<4>(ln.gamma + goff[e], gq);
             load_cells<4>(ln.beta + goff[e], bq);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {  // zeros outside the grid: no test per element then
+                gq[c] = ok[e] ? gq[c] : 0.f;
+                bq[c] = ok[e] ? bq[c] : 0.f;
+            }
             store_cells<4>(gam_rows + loff[e], gq);
             store_cells<4>(bet_rows + loff[e], bq);
         }
@@ -153,7 +158,7 @@ void bwd_rows(const float *__restrict__ weight, const float *__restrict__ bias, 
                 load_cells<4>(gam_rows + loff[e], gq);
                 load_cells<4>(bet_rows + loff[e], bq);
 #pragma unroll
-                for (int q = 0; q < 4; ++q) v[q] = ok[e] ? fmaf((xbuf[e][q] - xmean) * xrstd, gq[q], bq[q]) : 0.f;
+                for (int q = 0; q < 4; ++q) v[q] = fmaf((xbuf[e][q] - xmean) * xrstd, gq[q], bq[q]);
             } else {
 #pragma unroll
                 for (int q = 0; q < 4; ++q) v[q] = ok[e] ? xbuf[e][q] : 0.f;

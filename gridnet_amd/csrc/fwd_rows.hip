@@ -49,7 +49,6 @@ void fwd_rows(const float *__restrict__ weight, const float *__restrict__ bias, 
     const int nbj = N / kRowsTube, p0 = (tube / nbj) * kRowsTube, q0 = (tube % nbj) * kRowsTube;
     const long cells = (long)M * N * K;
     const int grow = ((p0 + ci) * N + (q0 + cj)) * K + 4 * bk;  // this thread's four cells
-    const bool first = bk == 0, last = bk == kb - 1;
     const bool ln_in = LN && ln.x_stats != nullptr;  // x is the raw output of the step before
 
     float w[9][3][4], bv[4], rv[4];
@@ -59,6 +58,14 @@ void fwd_rows(const float *__restrict__ weight, const float *__restrict__ bias, 
         for (int cc = 0; cc < 3; ++cc) load_cells<4>(weight + (pq * 3 + cc) * cells + grow, w[pq][cc]);
     load_cells<4>(bias + grow, bv);
     load_cells<4>(scale + grow, rv);
+    // the taps that would leave the row along K: their weights are zeroed instead of the value the
+    // neighbouring lane (a piece of another row) sends
+    const float keep_first = bk == 0 ? 0.f : 1.f, keep_last = bk == kb - 1 ? 0.f : 1.f;
+#pragma unroll
+    for (int pq = 0; pq < 9; ++pq) {
+        w[pq][0][0] *= keep_first;
+        w[pq][2][3] *= keep_last;
+    }
 
     // ---- the rows this thread moves: rows r, r + 16 and (the first four r) r + 32 ----
     int goff[kRowsRpt], loff[kRowsRpt];
@@ -71,10 +78,17 @@ void fwd_rows(const float *__restrict__ weight, const float *__restrict__ bias, 
         ok[e] = row < kRowsWin && gi >= 0 && gi < M && gj >= 0 && gj < N;
         goff[e] = ok[e] ? (gi * N + gj) * K + 4 * bk : grow;  // anything valid when not used
         loff[e] = row * K + 4 * bk;
-        if (ln_in && row < kRowsWin) {  // gamma and beta of the row, once per workgroup
+        if (ln_in && row < kRowsWin) {
+            // gamma and beta of the row, once per workgroup; zeros for a row outside the grid, which
+            // makes whatever is loaded in its place a zero without a test per element
             float gq[4], bq[4];
             load_cells<4>(ln.gamma + goff[e], gq);
             load_cells<4>(ln.beta + goff[e], bq);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                gq[q] = ok[e] ? gq[q] : 0.f;
+                bq[q] = ok[e] ? bq[q] : 0.f;
+            }
             store_cells<4>(gam_rows + loff[e], gq);
             store_cells<4>(bet_rows + loff[e], bq);
         }
@@ -107,7 +121,7 @@ void fwd_rows(const float *__restrict__ weight, const float *__restrict__ bias, 
                 load_cells<4>(gam_rows + loff[e], gq);
                 load_cells<4>(bet_rows + loff[e], bq);
 #pragma unroll
-                for (int q = 0; q < 4; ++q) v[q] = ok[e] ? fmaf((xbuf[e][q] - xmean) * xrstd, gq[q], bq[q]) : 0.f;
+                for (int q = 0; q < 4; ++q) v[q] = fmaf((xbuf[e][q] - xmean) * xrstd, gq[q], bq[q]);
             } else {
 #pragma unroll
                 for (int q = 0; q < 4; ++q) v[q] = ok[e] ? xbuf[e][q] : 0.f;
@@ -119,6 +133,9 @@ void fwd_rows(const float *__restrict__ weight, const float *__restrict__ bias, 
         for (int c = 0; c < 4; ++c) base[c] = RES ? raw[c] : 0.f;
         lds_barrier();  // the stage is complete (the first: gamma and beta too); the other one's readers are done
         fetch(min(s + 1, s1 - 1));
+        // the requests leave now, with the whole stencil in front of the element that needs them
+        // (left to itself the compiler sinks two of the three past it)
+        __builtin_amdgcn_sched_barrier(0);
         float u[4], own[4];
 #pragma unroll
         for (int c = 0; c < 4; ++c) u[c] = bv[c];
@@ -128,9 +145,8 @@ void fwd_rows(const float *__restrict__ weight, const float *__restrict__ bias, 
             const int di = pq / 3 - 1, dj = pq % 3 - 1;
             float d[6], mid[4];
             load_cells<4>(stage + (own_row + di * (kRowsTube + 2) + dj) * K + 4 * bk, mid);
-            const float before = lane_before(mid[3]), after = lane_after(mid[0]);
-            d[0] = first ? 0.f : before;
-            d[5] = last ? 0.f : after;
+            d[0] = lane_before(mid[3]);
+            d[5] = lane_after(mid[0]);
 #pragma unroll
             for (int c = 0; c < 4; ++c) d[c + 1] = mid[c];
             if (pq == 4) {

@@ -11,7 +11,7 @@ import torch
 
 from oracle.network import network_forward, network_forward_backward
 
-from helpers import assert_close, inputs_clear_of_kink
+from helpers import assert_chain_close, assert_close, inputs_clear_of_kink
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -75,8 +75,7 @@ def test_fused_chain_matches_oracle(name, grid, batch, outer, activation):
         return t
 
     t = inputs_clear_of_kink(wl, make)
-    for name_, got, exp in zip(NAMES, run_fused(wl, t, True), oracle(wl, t, True)):
-        assert_close(got, exp, what=name_)
+    assert_chain_close(NAMES, run_fused(wl, t, True), oracle(wl, t, True), t, wl)
 
 
 @pytest.mark.parametrize("name,grid,batch,outer", [("C2", 32, 4, 3), ("C4", 32, 2, 2)])

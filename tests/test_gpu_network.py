@@ -8,7 +8,7 @@ import torch
 
 from oracle.network import network_forward_backward, network_forward
 
-from helpers import assert_close, inputs_clear_of_kink
+from helpers import assert_chain_close, assert_close, inputs_clear_of_kink
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -40,8 +40,7 @@ def check_against_oracle(wl, t, backward):
     want = network_forward_backward([t[k].double() for k in PARAMS], t["x0"].double(),
                                     t["grad_out"].double(), **kw)
     names = ("y", "dweight", "dbias", "dscale", "dgamma", "dbeta", "dx0")
-    for name, got, exp in zip(names, (y, *grads), want):
-        assert_close(got, exp, what=name)
+    assert_chain_close(names, (y, *grads), want, t, wl)
 
 
 def test_c1_exact_config_forward_and_backward():

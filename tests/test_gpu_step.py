@@ -280,3 +280,40 @@ def test_machine_ceiling_probes_report_sane_figures():
     assert widths["ds_read_b32"] < widths["ds_read_b128"]
     with pytest.raises(RuntimeError, match="unknown"):
         p.probe_id(99)
+
+
+@pytest.mark.parametrize("activation", ["silu", "tanh"])
+@pytest.mark.parametrize("shape,bs,inner", [((8, 8, 32), 4, 1), ((8, 8, 8), 8, 2), ((8, 8, 8), 4, 3)])
+def test_smooth_activations_to_a_few_ulp(activation, shape, bs, inner):
+    """The activation and its derivative on their own: with all weights zero every inner iteration
+    sees the pre-activation u = bias, so y = x + inner*act(bias) and dbias = inner*act'(bias) for
+    residual_scale = 1 and an incoming gradient of ones.  Pre-activations from -100 to 100, dense
+    around 0: the kernels' fp32 silu (exp2 and reciprocal instructions with a compensated
+    argument) and tanh must stay within a few units in the last place of the fp64 value, where
+    the bar of the parity tests (1e-4 relative) would hide a sloppy exponential."""
+    n = shape[0] * shape[1] * shape[2]
+    g = torch.Generator().manual_seed(5)
+    u = torch.cat([torch.linspace(-100, 100, n // 2), 8 * torch.randn(n - n // 2, generator=g)]).float()
+    u[:8] = torch.tensor([0.0, -0.0, 1e-30, -1e-30, 87.5, -87.5, 103.9, -103.9])
+    b = u.reshape(shape)
+    w, r, x = torch.zeros(27, *shape), torch.ones(shape), torch.zeros(1, *shape)
+    y, grads = run_op(w, b, r, x, torch.ones(1, *shape), inner, bs, 1e-5, False, activation)
+    ud = b.double()
+    if activation == "silu":
+        s = torch.sigmoid(ud)
+        f, d = ud * s, s * (1 + ud * (1 - s))
+    else:
+        f = torch.tanh(ud)
+        d = 1 - f * f
+    ulp = 2.0 ** -23
+    # 4 ulp of the value.  silu' = s (1 + u (1 - s)) takes 1 - s from an s that is rounded to
+    # fp32: 2^-24 |u| s of absolute error comes with the formula, whatever exponential is behind it
+    # tanh is formed as (1 - e) / (1 + e), a difference of numbers near 1 when u is near 0 (the
+    # reference's 2 sigmoid(2u) - 1, src/activations.h:130, is one too): absolute there
+    floor = 2 * ulp if activation == "tanh" else 1e-30
+    assert_close(y[0].double() / inner, f, rtol=4 * ulp, atol=floor, what=f"{activation}(u)")
+    err = (grads[1].double() / inner - d).abs()
+    bound = 4 * ulp * d.abs() + floor
+    if activation == "silu":
+        bound = bound + 2 * ulp * ud.abs() * s
+    assert bool((err <= bound).all()), f"{activation}'(u): worst excess {(err - bound).max().item():.3e}"
