@@ -64,7 +64,6 @@ void bwd_rows(const float *__restrict__ weight, const float *__restrict__ bias, 
     const int nbj = N / kTube, p0 = (tube / nbj) * kTube, q0 = (tube % nbj) * kTube;
     const long cells = (long)M * N * K;
     const int grow = ((p0 + ci) * N + (q0 + cj)) * K + 2 * bk;  // this thread's two cells
-    const bool first = bk == 0, last = bk == kb - 1;
     const bool ln_in = LN && ln.x_stats != nullptr;              // x is the raw output of the step before
     const bool through_ln = LN && (!RES || ln.y_raw != nullptr);  // dy passes a LayerNorm on load
 
@@ -78,6 +77,14 @@ void bwd_rows(const float *__restrict__ weight, const float *__restrict__ bias, 
     load_cells<2>(bias + grow, bv);
     load_cells<2>(scale + grow, rv);
     if (LN) load_cells<2>(ln.gamma + grow, gam);
+    // The taps that would leave the row along K read what the neighbouring lane sends, a piece of
+    // another row: their weights are zeroed here, and their weight gradients at the end.
+    const float keep_first = bk == 0 ? 0.f : 1.f, keep_last = bk == kb - 1 ? 0.f : 1.f;
+#pragma unroll
+    for (int pq = 0; pq < 9; ++pq) {
+        w[pq * 3][0] *= keep_first;
+        w[pq * 3 + 2][1] *= keep_last;
+    }
 
     // ---- the window rows this thread moves, as 16-byte pieces: piece tid and, for the first
     // eighth of the threads, piece tid + nt (36 K / 4 pieces in all) ----
@@ -110,20 +117,6 @@ void bwd_rows(const float *__restrict__ weight, const float *__restrict__ bias, 
     }
     const int own_row = (ci + 1) * (kTube + 2) + (cj + 1);
     wait_global_loads();
-    // Add-in-place mode: the accumulators start from what the gradient buffers hold (requested
-    // behind the set-up wait, arriving during the first element) and are stored at the end like in
-    // the overwrite mode.
-    if (param_mode == kParamAddExclusive) {
-#pragma unroll
-        for (int t = 0; t < 27; ++t) load_cells<2>(dweight + t * cells + grow, nw[t]);
-        load_cells<2>(dbias + grow, db);
-        load_cells<2>(dscale + grow, dr);
-        if (LN) {
-            load_cells<2>(ln.dgamma + grow, dgam);
-            load_cells<2>(ln.dbeta + grow, dbet);
-        }
-    }
-
     const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
     float xbuf[2][4], gnext[2], ynext[2] = {0.f, 0.f}, gprev[2] = {0.f, 0.f}, dxold[2] = {0.f, 0.f};
     float xmean = 0.f, xrstd = 1.f, ny[4] = {0.f, 1.f, 0.f, 0.f};
@@ -191,11 +184,10 @@ void bwd_rows(const float *__restrict__ weight, const float *__restrict__ bias, 
                 const int di = pq / 3 - 1, dj = pq % 3 - 1;
                 float mid[2], d[4];
                 load_cells<2>(stage + (own_row + di * (kTube + 2) + dj) * K + 2 * bk, mid);
-                const float before = lane_before(mid[1]), after = lane_after(mid[0]);
-                d[0] = first ? 0.f : before;
+                d[0] = lane_before(mid[1]);
                 d[1] = mid[0];
                 d[2] = mid[1];
-                d[3] = last ? 0.f : after;
+                d[3] = lane_after(mid[0]);
                 use(pq, d);
             }
         };
@@ -229,6 +221,27 @@ void bwd_rows(const float *__restrict__ weight, const float *__restrict__ bias, 
         });
     }
     // ---- parameter gradients: plain stores of whole rows ----
+#pragma unroll
+    for (int pq = 0; pq < 9; ++pq) {
+        nw[pq * 3][0] *= keep_first;
+        nw[pq * 3 + 2][1] *= keep_last;
+    }
+    if (param_mode == kParamAddExclusive) {  // add-in-place mode: on top of what the buffers hold
+        auto add_old = [&](const float *from, float (&v)[2]) {
+            float old[2];
+            load_cells<2>(from + grow, old);
+            v[0] += old[0];
+            v[1] += old[1];
+        };
+#pragma unroll
+        for (int t = 0; t < 27; ++t) add_old(dweight + t * cells, nw[t]);
+        add_old(dbias, db);
+        add_old(dscale, dr);
+        if (LN) {
+            add_old(ln.dgamma, dgam);
+            add_old(ln.dbeta, dbet);
+        }
+    }
 #pragma unroll
     for (int t = 0; t < 27; ++t) store_cells<2>(dweight + t * cells + grow, nw[t]);
     store_cells<2>(dbias + grow, db);
