@@ -333,7 +333,14 @@ static size_t fused_backward_dsum(const StepArgs &a) {
 }
 static size_t fused_backward_parts(const StepArgs &a) {
     const size_t nblk = (size_t)(a.M / a.block_size) * (a.N / a.block_size) * (a.K / a.block_size);
-    return (size_t)a.B * nblk * step_fast_backward_parts(a.block_size) * 2 * sizeof(float);
+    size_t pairs = nblk * step_fast_backward_parts(a.block_size);
+    if (bwd_rows_supports(a)) {  // one inner iteration, by rows: a pair per wave of its first kernel
+        StepArgs plain = a;
+        plain.ln.residual = 0;
+        const size_t rows = (size_t)bwd_rows_pairs(plain);
+        if (rows > pairs) pairs = rows;
+    }
+    return (size_t)a.B * pairs * 2 * sizeof(float);
 }
 
 size_t gridnet_hip_fused_workspace_bytes(int B, int M, int N, int K, int inner, int block_size,
@@ -584,7 +591,7 @@ int gridnet_hip_chain_backward(int dtype, const void *weight, const void *bias, 
     // the sums come from chain_bwd itself (a pair per block) when dx is left unfinished, from the
     // cross-block kernel otherwise
     const int nblk = (M / block_size) * (N / block_size) * (K / block_size);
-    return layernorm_finalize_sums(a.ln.x_part, halo_out ? nblk : step_fast_backward_pairs(a),
+    return layernorm_finalize_sums(a.ln.x_part, halo_out ? nblk : step_fast_cross_pairs(a),
                                    (long)M * N * K, (float *)x_sums, B, st);
 }
 

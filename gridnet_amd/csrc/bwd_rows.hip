@@ -9,7 +9,17 @@
 // This kernel recomputes u, forms delta and the parameter gradients, and leaves delta of every cell
 // (in the scratch tensor the block kernels leave D in) and the direct part of dx, g.  The sum
 // over the neighbours' deltas is cross_rows' job (cross_rows.hip, with ALL taps instead of the
-// ones that cross a block boundary), which also forms the LayerNorm sums from the finished rows.
+// ones that cross a block boundary).
+//
+// The two sums the backward of the LayerNorm in FRONT of the step needs, sum gamma dx and
+// sum gamma dx xn (xn the normalised input before gamma and beta), are formed HERE, before dx
+// exists, so that cross_rows need not read x again: with xh = gamma xn + beta the step's input,
+//   sum_c gamma[c] dx[c]        = sum_c gamma[c] g[c] + delta[c] Wg[c],   Wg[c] = sum_t w[t, c] gamma[c + off_t]
+//   sum_c dx[c] (xh[c] - beta[c]) = sum_c g[c] (xh[c] - beta[c]) + delta[c] (u[c] - b[c] - Wb[c]),
+//                                                               Wb[c] = sum_t w[t, c] beta[c + off_t]
+// (every delta[c] reaches the cells c + off_t with the weights w[t, c], and sum_t w[t, c] xh[c + off_t]
+// is u[c] - b[c]); Wg and Wb are two numbers per cell, formed once per workgroup.  The residual
+// loop keeps cross_rows' sums.
 // The reference does all of this per block with shared-memory and global atomics
 // (src/gridnet_cuda_kernels.cu:300-450); here nothing is scattered.
 //
@@ -117,6 +127,33 @@ void bwd_rows(const float *__restrict__ weight, const float *__restrict__ bias, 
     }
     const int own_row = (ci + 1) * (kTube + 2) + (cj + 1);
     wait_global_loads();
+    // the LayerNorm sums of dx (see the head of the file): Wg and b + Wb of the thread's cells
+    const bool sums_here = LN && !RES && ln_in && ln.x_part != nullptr;
+    float bet[2] = {0.f, 0.f}, wgam[2] = {0.f, 0.f}, bwb[2] = {bv[0], bv[1]};
+    if (LN && !RES) {
+        if (sums_here) {  // the same for the whole workgroup
+            load_cells<2>(ln.beta + grow, bet);
+            __syncthreads();  // gamma and beta of the 36 rows are in LDS
+            auto over_taps = [&](const float *rows36, float (&acc)[2]) {
+#pragma unroll
+                for (int pq = 0; pq < 9; ++pq) {
+                    const int di = pq / 3 - 1, dj = pq % 3 - 1;
+                    float mid[2], d[4];
+                    load_cells<2>(rows36 + (own_row + di * (kTube + 2) + dj) * K + 2 * bk, mid);
+                    d[0] = lane_before(mid[1]);
+                    d[1] = mid[0];
+                    d[2] = mid[1];
+                    d[3] = lane_after(mid[0]);
+#pragma unroll
+                    for (int cc = 0; cc < 3; ++cc)
+#pragma unroll
+                        for (int c = 0; c < 2; ++c) acc[c] = fmaf(w[pq * 3 + cc][c], d[c + cc], acc[c]);
+                }
+            };
+            over_taps(gam_rows, wgam);
+            over_taps(bet_rows, bwb);
+        }
+    }
     const int s0 = chunk * chunk_len, s1 = min(B, s0 + chunk_len);
     float xbuf[2][4], gnext[2], ynext[2] = {0.f, 0.f}, gprev[2] = {0.f, 0.f}, dxold[2] = {0.f, 0.f};
     float xmean = 0.f, xrstd = 1.f, ny[4] = {0.f, 1.f, 0.f, 0.f};
@@ -191,8 +228,12 @@ void bwd_rows(const float *__restrict__ weight, const float *__restrict__ bias, 
                 use(pq, d);
             }
         };
-        float u[2] = {bv[0], bv[1]};
+        float u[2] = {bv[0], bv[1]}, own[2] = {0.f, 0.f};
         rows([&](int pq, const float (&d)[4]) {
+            if (pq == 4) {
+                own[0] = d[1];
+                own[1] = d[2];
+            }
 #pragma unroll
             for (int cc = 0; cc < 3; ++cc)
 #pragma unroll
@@ -213,6 +254,22 @@ void bwd_rows(const float *__restrict__ weight, const float *__restrict__ bias, 
         store_cells<2>(delta_out + o, delta);
         store_cells<2>(dx + o, out);
         if (RES && ln.g_out) store_cells<2>(ln.g_out + o, gin);
+        if (LN && !RES) {
+            if (sums_here) {
+                float t1 = 0.f, t2 = 0.f;
+#pragma unroll
+                for (int c = 0; c < 2; ++c) {
+                    t1 = fmaf(gam[c], out[c], fmaf(delta[c], wgam[c], t1));
+                    t2 = fmaf(out[c], own[c] - bet[c], fmaf(delta[c], u[c] - bwb[c], t2));
+                }
+                const float w1 = slot_wave_sum<64>(t1), w2 = slot_wave_sum<64>(t2);
+                if ((tid & 63) == 0) {
+                    float *to = ln.x_part + (((long)s * ntube + tube) * (nt / 64) + tid / 64) * 2;
+                    to[0] = w1;
+                    to[1] = w2;
+                }
+            }
+        }
         rows([&](int pq, const float (&d)[4]) {
 #pragma unroll
             for (int cc = 0; cc < 3; ++cc)
@@ -306,8 +363,9 @@ template <int ACT, bool LN, bool RES> int launch(const StepArgs &a, hipStream_t 
         if (int rc = plan_reduce_slabs(slab, nchunk, slab_floats, t, new_params ? 0 : 1, st)) return rc;
     }
     // dx holds its direct part, the scratch tensor delta: the sum over the neighbours' deltas, all
-    // 27 taps of it, and with the LayerNorm folded in the sums of the finished rows
-    return cross_rows_full_launch(a, st);
+    // 27 taps of it; the LayerNorm sums of the finished rows only where the kernel above left them out
+    const bool sums_here = LN && !RES && a.ln.x_stats && a.ln.x_part;
+    return cross_rows_full_launch(a, st, !sums_here);
 }
 
 template <int ACT> int dispatch(const StepArgs &a, hipStream_t st) {
@@ -321,6 +379,11 @@ template <int ACT> int dispatch(const StepArgs &a, hipStream_t st) {
 bool bwd_rows_supports(const StepArgs &a) {
     return a.dtype == GRIDNET_F32 && a.inner == 1 && !a.normalize && (a.block_size == 4 || a.block_size == 8) &&
            k_ok(a.K) && a.M % 4 == 0 && a.N % 4 == 0 && cross_rows_supports(a);
+}
+
+int bwd_rows_pairs(const StepArgs &a) {
+    if (a.ln.residual) return cross_rows_pairs(a);
+    return (a.M / kTube) * (a.N / kTube) * (8 * a.K / 64);
 }
 
 // room for per-chunk copies of the gradient arrays that lets the batch be split as far as the

@@ -322,9 +322,10 @@ int cross_rows_launch(const StepArgs &a, hipStream_t st) {
 }
 
 // all 27 taps (the second kernel of bwd_rows.hip); the block size does not enter then
-int cross_rows_full_launch(const StepArgs &a, hipStream_t st) {
+int cross_rows_full_launch(const StepArgs &a, hipStream_t st, bool ln_sums) {
     const float *dsum = (const float *)a.workspace;
-    return a.ln.gamma ? launch<4, true, false, 1, true>(a, dsum, st) : launch<4, false, false, 1, true>(a, dsum, st);
+    return a.ln.gamma && ln_sums ? launch<4, true, false, 1, true>(a, dsum, st)
+                                 : launch<4, false, false, 1, true>(a, dsum, st);
 }
 
 // the gated update: weight [27, 2, M, N, K], D0 and D1 of every cell behind one another in `dsum`

@@ -109,6 +109,7 @@ int step_fast_forward_pairs(const StepArgs &a);       // pairs per sample that t
 int step_fast_forward_pair_count(const StepArgs &a);  // ... and the cells behind each
 int step_fast_backward_parts(int block_size);  // (sum g, sum g*xhat) pairs per (block, element), at most
 int step_fast_backward_pairs(const StepArgs &a);  // pairs per sample that the backward of `a` leaves
+int step_fast_cross_pairs(const StepArgs &a);     // the same for step_cross_launch alone (behind chain_bwd)
 
 // fwd_rows.hip: the forward of a step with ONE inner iteration, dealt by whole K-rows (fp32, normalize
 // off, K of 16, 32, 64 or 128; the folded LayerNorm and the residual form as a.ln says)
@@ -122,6 +123,9 @@ int fwd_rows_launch(const StepArgs &a, hipStream_t st);
 bool bwd_rows_supports(const StepArgs &a);
 size_t bwd_rows_slab_bytes(const StepArgs &a);
 int bwd_rows_launch(const StepArgs &a, hipStream_t st);
+// LayerNorm sum pairs per sample in a.ln.x_part after bwd_rows_launch (the plain loop: the first
+// kernel forms them, one pair per wave; the residual loop: cross_rows_pairs)
+int bwd_rows_pairs(const StepArgs &a);
 
 // cross_rows.hip: the cross-block part of the backward for 4^3 blocks, dealt by whole K-rows
 // (a.workspace holds D, a.dx the block-local part; LayerNorm fold as a.ln says); K of 16, 32, 64
@@ -129,7 +133,8 @@ int bwd_rows_launch(const StepArgs &a, hipStream_t st);
 bool cross_rows_supports(const StepArgs &a);
 int cross_rows_pairs(const StepArgs &a);  // LayerNorm sum pairs per sample that it leaves in a.ln.x_part
 int cross_rows_launch(const StepArgs &a, hipStream_t st);
-int cross_rows_full_launch(const StepArgs &a, hipStream_t st);  // all 27 taps, for bwd_rows.hip
+// all 27 taps, for bwd_rows.hip; ln_sums: with the LayerNorm sums of the finished rows (a.ln.x_part)
+int cross_rows_full_launch(const StepArgs &a, hipStream_t st, bool ln_sums);
 bool cross_rows_gated_supports(const StepArgs &a);  // the gated update: two weight sets, D0 and D1 in `dsum`
 int cross_rows_gated_launch(const StepArgs &a, const float *dsum, hipStream_t st);
 

@@ -1916,6 +1916,10 @@ int step_fast_forward_pair_count(const StepArgs &a) {
 }
 int step_fast_backward_parts(int block_size) { return block_size == 8 ? 2 : 1; }
 int step_fast_backward_pairs(const StepArgs &a) {
+    if (bwd_rows_supports(a)) return bwd_rows_pairs(a);
+    return step_fast_cross_pairs(a);
+}
+int step_fast_cross_pairs(const StepArgs &a) {
     if (cross_rows_supports(a)) return cross_rows_pairs(a);
     return (a.M / a.block_size) * (a.N / a.block_size) * (a.K / a.block_size);
 }
