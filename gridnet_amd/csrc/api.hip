@@ -492,8 +492,9 @@ static int fused_backward(int dtype, const void *weight, const void *bias, const
     a.ln.residual = residual;
     a.ln.g_prev = (const float *)g_prev;
     a.ln.g_out = (float *)g_out;
+    a.ln.x_sums = (float *)x_sums;
     if (int rc = step_backward_fast(a, st)) return rc;
-    if (!x_stats) return GRIDNET_OK;
+    if (!x_stats || bwd_rows_leaves_sums(a)) return GRIDNET_OK;
     return layernorm_finalize_sums(a.ln.x_part, step_fast_backward_pairs(a),
                                    (long)M * N * K, (float *)x_sums, B, st);
 }

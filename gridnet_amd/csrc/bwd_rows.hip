@@ -360,7 +360,12 @@ template <int ACT, bool LN, bool RES> int launch(const StepArgs &a, hipStream_t 
             t.dst[4] = a.ln.dbeta;  t.end[4] = 31 * cells;
             t.count = 5;
         }
-        if (int rc = plan_reduce_slabs(slab, nchunk, slab_floats, t, new_params ? 0 : 1, st)) return rc;
+        // the LayerNorm sums the kernel above left per wave are finished by spare workgroups of this one
+        SumsJob job{nullptr, 0, 0, 0, nullptr};
+        if (bwd_rows_leaves_sums(a)) job = SumsJob{a.ln.x_part, bwd_rows_pairs(a), a.B, cells, a.ln.x_sums};
+        if (int rc = plan_reduce_slabs(slab, nchunk, slab_floats, t, new_params ? 0 : 1, st, job)) return rc;
+    } else if (bwd_rows_leaves_sums(a)) {
+        if (int rc = layernorm_finalize_sums(a.ln.x_part, bwd_rows_pairs(a), cells, a.ln.x_sums, a.B, st)) return rc;
     }
     // dx holds its direct part, the scratch tensor delta: the sum over the neighbours' deltas, all
     // 27 taps of it; the LayerNorm sums of the finished rows only where the kernel above left them out
@@ -379,6 +384,10 @@ template <int ACT> int dispatch(const StepArgs &a, hipStream_t st) {
 bool bwd_rows_supports(const StepArgs &a) {
     return a.dtype == GRIDNET_F32 && a.inner == 1 && !a.normalize && (a.block_size == 4 || a.block_size == 8) &&
            k_ok(a.K) && a.M % 4 == 0 && a.N % 4 == 0 && cross_rows_supports(a);
+}
+
+bool bwd_rows_leaves_sums(const StepArgs &a) {
+    return bwd_rows_supports(a) && a.ln.gamma && !a.ln.residual && a.ln.x_stats && a.ln.x_part && a.ln.x_sums;
 }
 
 int bwd_rows_pairs(const StepArgs &a) {

@@ -120,6 +120,49 @@ template <typename T> __device__ __forceinline__ T block_sum(T v, T *scratch, in
     return total;
 }
 
+// ---- device: the last step of the LayerNorm backward's two sums --------------------------
+// (s1_i, s2_i), `parts` pairs of sample b -> (sum s1 / n, sum s2 / n), by one workgroup of THREADS
+// threads: doubles, a fixed order.  `red` is LDS, one pair per wave.  A kernel of its own in
+// layernorm.hip; also run by spare workgroups of the kernel that adds up the gradient copies.
+constexpr int kFinUnroll = 4;  // pairs a thread requests before it uses any
+template <int THREADS>
+__device__ __forceinline__ void finalize_sums_of_sample(const float *__restrict__ part, int parts, long n,
+                                                        float *__restrict__ sums, int b,
+                                                        double (*red)[2]) {
+    const int tid = threadIdx.x;
+    const float2 *ps = reinterpret_cast<const float2 *>(part) + (long)b * parts;
+    double s1 = 0.0, s2 = 0.0;
+    for (int i0 = tid; i0 < parts; i0 += THREADS * kFinUnroll) {
+        float2 v[kFinUnroll];
+#pragma unroll
+        for (int k = 0; k < kFinUnroll; ++k) {
+            const int i = i0 + k * THREADS;
+            v[k] = i < parts ? ps[i] : make_float2(0.f, 0.f);
+        }
+#pragma unroll
+        for (int k = 0; k < kFinUnroll; ++k) {
+            s1 += (double)v[k].x;
+            s2 += (double)v[k].y;
+        }
+    }
+    s1 = wave_sum(s1);
+    s2 = wave_sum(s2);
+    if ((tid & (kWave - 1)) == 0) {
+        red[tid / kWave][0] = s1;
+        red[tid / kWave][1] = s2;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        s1 = s2 = 0.0;
+        for (int w = 0; w < THREADS / kWave; ++w) {
+            s1 += red[w][0];
+            s2 += red[w][1];
+        }
+        sums[2 * b] = (float)(s1 / (double)n);
+        sums[2 * b + 1] = (float)(s2 / (double)n);
+    }
+}
+
 // ---- device: gathering what a block's cells send to the window around it -----------------
 // In the backward of a block-local update every cell c sends weight[t][c] * delta[c] to window
 // entry c + offset(t), t = 9a+3b+c' <-> offset (a-1, b-1, c'-1).  Scattering that with LDS float

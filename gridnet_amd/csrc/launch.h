@@ -24,6 +24,8 @@ struct LnFold {
     const float *y_sums;        // [B,2]: mean(g), mean(g * yhat) with g = gamma * incoming gradient
     float *dgamma, *dbeta;      // [M,N,K], summed over the batch, committed like dbias
     float *x_part;              // partial sums for the LayerNorm backward of x: [B, nblk, parts, 2]
+    float *x_sums;              // [B,2] or null: where a backward that finishes the sums itself leaves them
+                                // (bwd_rows_leaves_sums); otherwise the caller finalizes x_part
     // The reference's outer_residual form of the loop (gridnet/scripts/train_imagenet.py:81-83):
     // h' = h + (step(n) - n), n = LayerNorm(h).  Forward: the output is x + (result - n); needs
     // x_stats.  Backward of the step that produced h' from h = x, with G' the gradient with
@@ -126,6 +128,8 @@ int bwd_rows_launch(const StepArgs &a, hipStream_t st);
 // LayerNorm sum pairs per sample in a.ln.x_part after bwd_rows_launch (the plain loop: the first
 // kernel forms them, one pair per wave; the residual loop: cross_rows_pairs)
 int bwd_rows_pairs(const StepArgs &a);
+// bwd_rows_launch leaves a.ln.x_sums finished (no finalize call behind it)
+bool bwd_rows_leaves_sums(const StepArgs &a);
 
 // cross_rows.hip: the cross-block part of the backward for 4^3 blocks, dealt by whole K-rows
 // (a.workspace holds D, a.dx the block-local part; LayerNorm fold as a.ln says); K of 16, 32, 64

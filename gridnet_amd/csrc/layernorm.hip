@@ -277,7 +277,6 @@ __global__ __launch_bounds__(kLnThreads) void ln_bwd_apply(
 // The step kernels leave per-group partial results; these small kernels turn them into the
 // per-sample numbers, in double and in a fixed order (one workgroup per sample).
 
-constexpr int kFinUnroll = 4;  // pairs a thread requests before it uses any
 // workgroup size: as few waves as request every pair in one round (fewer waves start sooner and
 // leave a shorter last loop), up to the largest workgroup
 inline int finalize_threads(int parts) {
@@ -342,38 +341,7 @@ __global__ __launch_bounds__(THREADS) void ln_finalize_sums(const float *__restr
                                                                 int parts, long n,
                                                                 float *__restrict__ sums) {
     __shared__ double red[THREADS / kWave][2];
-    const int tid = threadIdx.x, b = blockIdx.x;
-    const float2 *ps = reinterpret_cast<const float2 *>(part) + (long)b * parts;
-    double s1 = 0.0, s2 = 0.0;
-    for (int i0 = tid; i0 < parts; i0 += THREADS * kFinUnroll) {
-        float2 v[kFinUnroll];
-#pragma unroll
-        for (int k = 0; k < kFinUnroll; ++k) {
-            const int i = i0 + k * THREADS;
-            v[k] = i < parts ? ps[i] : make_float2(0.f, 0.f);
-        }
-#pragma unroll
-        for (int k = 0; k < kFinUnroll; ++k) {
-            s1 += (double)v[k].x;
-            s2 += (double)v[k].y;
-        }
-    }
-    s1 = wave_sum(s1);
-    s2 = wave_sum(s2);
-    if ((tid & (kWave - 1)) == 0) {
-        red[tid / kWave][0] = s1;
-        red[tid / kWave][1] = s2;
-    }
-    __syncthreads();
-    if (tid == 0) {
-        s1 = s2 = 0.0;
-        for (int w = 0; w < THREADS / kWave; ++w) {
-            s1 += red[w][0];
-            s2 += red[w][1];
-        }
-        sums[2 * b] = (float)(s1 / (double)n);
-        sums[2 * b + 1] = (float)(s2 / (double)n);
-    }
+    finalize_sums_of_sample<THREADS>(part, parts, n, sums, blockIdx.x, red);
 }
 
 // y = (x - mean) * rstd * gamma + beta with statistics that are already known
