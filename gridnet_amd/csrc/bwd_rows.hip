@@ -161,7 +161,7 @@ void bwd_rows(const float *__restrict__ weight, const float *__restrict__ bias, 
         const long at = (long)s * cells;
         load_cells<2>(dy + at + grow, gnext);
         if (through_ln) {
-            load_cells<2>(ln.y_raw + at + grow, ynext);
+            if (RES) load_cells<2>(ln.y_raw + at + grow, ynext);  // the plain loop recomputes it
             ny[0] = load_ahead(ln.y_stats, 2 * s);
             ny[1] = load_ahead(ln.y_stats, 2 * s + 1);
             ny[2] = load_ahead(ln.y_sums, 2 * s);
@@ -196,10 +196,15 @@ void bwd_rows(const float *__restrict__ weight, const float *__restrict__ bias, 
             store_cells<4>(stage + loff[e], v);
         }
         // the element's incoming gradient, through the backward of the LayerNorm behind the step
-        float g[2], gin[2];
+        // (the plain loop: further down, from the raw output recomputed there; what the prefetch of the
+        // next element is about to overwrite is set aside)
+        constexpr bool kLate = LN && !RES;
+        float g[2], gin[2], gcur[2] = {gnext[0], gnext[1]}, nyc[4] = {ny[0], ny[1], ny[2], ny[3]};
 #pragma unroll
         for (int c = 0; c < 2; ++c) {
-            if (through_ln) {
+            if (kLate) {
+                g[c] = 0.f;
+            } else if (through_ln) {
                 const float yh = (ynext[c] - ny[0]) * ny[1];
                 dgam[c] = fmaf(gnext[c], yh, dgam[c]);
                 dbet[c] += gnext[c];
@@ -244,6 +249,14 @@ void bwd_rows(const float *__restrict__ weight, const float *__restrict__ bias, 
         for (int c = 0; c < 2; ++c) {
             float f, d;
             Act<ACT, float>::fd(u[c], f, d);
+            if (kLate) {
+                // the step's raw output as the forward formed it (fwd_rows.hip: the same multiply-adds in
+                // the same order), instead of reading it back: a quarter of this kernel's reads
+                const float yh = (fmaf(rv[c], f, own[c]) - nyc[0]) * nyc[1];
+                dgam[c] = fmaf(gcur[c], yh, dgam[c]);
+                dbet[c] += gcur[c];
+                g[c] = nyc[1] * (gam[c] * gcur[c] - nyc[2] - yh * nyc[3]);
+            }
             delta[c] = d * g[c] * rv[c];
             dr[c] = fmaf(f, g[c], dr[c]);
             db[c] += delta[c];
