@@ -374,10 +374,11 @@ def test_fused_forward_flags_match_the_plain_entry_points(bs, shape, batch):
         call(n.lib.gridnet_hip_fused_forward_flags, 4)
 
 
-@pytest.mark.parametrize("shape,bs,batch,residual", [
-    ((8, 12, 16), 4, 3, False), ((16, 8, 32), 8, 9, False), ((8, 16, 64), 8, 5, True), ((4, 8, 128), 4, 2, True),
-    ((16, 16, 32), 8, 20, False)])
-def test_fused_chain_with_one_inner_iteration(shape, bs, batch, residual):
+@pytest.mark.parametrize("shape,bs,batch,residual,activation", [
+    ((8, 12, 16), 4, 3, False, "silu"), ((16, 8, 32), 8, 9, False, "silu"), ((8, 16, 64), 8, 5, True, "silu"),
+    ((4, 8, 128), 4, 2, True, "silu"), ((16, 16, 32), 8, 20, False, "silu"),
+    ((16, 16, 32), 8, 17, False, "tanh"), ((8, 12, 16), 4, 3, False, "leaky_relu"), ((8, 8, 64), 8, 16, True, "tanh")])
+def test_fused_chain_with_one_inner_iteration(shape, bs, batch, residual, activation):
     """inner_iterations = 1 (the default of the reference's MNIST script,
     gridnet/scripts/train_mnist.py:77): the forward is a plain stencil over the whole grid and goes by
     whole K-rows (csrc/fwd_rows.hip), with the LayerNorm folded in and in both shapes of the loop;
@@ -386,7 +387,7 @@ def test_fused_chain_with_one_inner_iteration(shape, bs, batch, residual):
     from helpers import make_acts, make_params
 
     inner, outer = 1, 3
-    print(f"fused chain, one inner iteration: shape={shape} bs={bs} batch={batch} residual={residual}", flush=True)
+    print(f"fused chain, one inner iteration: shape={shape} bs={bs} batch={batch} residual={residual} act={activation}", flush=True)
     w, b, r = make_params(shape, seed=51)
     if residual:
         w, r = w * 0.5, r * 0.5
@@ -395,17 +396,17 @@ def test_fused_chain_with_one_inner_iteration(shape, bs, batch, residual):
     beta = 0.2 * torch.randn(shape, generator=g)
     x0, gy = make_acts(batch, shape, seed=53), make_acts(batch, shape, seed=54)
     run = BodyRunner(*(v.to(DEV) for v in (w, b, r, gamma, beta)), batch, inner, outer, bs,
-                     "silu", False, backward=True, fused=True, outer_residual=residual)
+                     activation, False, backward=True, fused=True, outer_residual=residual)
     y = run.forward(x0.to(DEV)).clone()
     got = (y, *[v.clone() for v in run.backward(gy.to(DEV))])
     exp = network_forward_backward([v.double() for v in (w, b, r, gamma, beta)], x0.double(),
                                    gy.double(), inner_iterations=inner, outer_iterations=outer,
-                                   block_size=bs, activation="silu", normalize=False,
+                                   block_size=bs, activation=activation, normalize=False,
                                    outer_residual=residual)
     summed = 1e-5 * max(1.0, (batch * inner * outer / 2) ** 0.5)
     for name_, a, e in zip(NAMES, got, exp):
         assert_close(a, e, atol=1e-5 if name_ in ("y", "dx0") else summed, what=name_)
     # forward only, with the walk alternating: the same bits
     fwd = BodyRunner(*(v.to(DEV) for v in (w, b, r, gamma, beta)), batch, inner, outer, bs,
-                     "silu", False, backward=False, fused=True, outer_residual=residual)
+                     activation, False, backward=False, fused=True, outer_residual=residual)
     assert torch.equal(fwd.forward(x0.to(DEV)), y)
