@@ -21,6 +21,7 @@
 
 #include "common.h"
 #include "launch.h"
+#include "plan.h"
 
 namespace gridnet {
 
@@ -410,7 +411,13 @@ template <typename T> int backward_t(const LayerNormArgs &a, hipStream_t st) {
                        block, 0, st, (const T *)a.dy, (const T *)a.x, (const T *)a.gamma,          \
                        (const T *)a.mean_in, (const T *)a.rstd_in, partial, nchunk, (T *)a.dx,     \
                        (T *)a.dgamma, (T *)a.dbeta, a.B, a.n)
-    if (vec) {
+    // A thread owns its cells for the whole batch, so the grid is n / (256 x cells per thread)
+    // workgroups whatever the batch: with four cells per thread a 32^3 grid is 32 of them (100 us
+    // at batch 256, 35 us with one cell per thread) and a 64^3 grid 256 (batch 128: 100 against
+    // 66 us; batch 32: 20 us either way).  Below two workgroups per CU a thread takes one cell:
+    // four times the workgroups, the same bits.
+    const bool wide = vec && a.n / (4L * kLnThreads) >= 2L * plan_device_cus();
+    if (wide) {
         if (accum) GRIDNET_LN_APPLY(4, true); else GRIDNET_LN_APPLY(4, false);
     } else {
         if (accum) GRIDNET_LN_APPLY(1, true); else GRIDNET_LN_APPLY(1, false);
